@@ -1,0 +1,136 @@
+"""Headline benchmark: FlashAttention forward TFLOPS on one MI355X, fp16, hd128, causal, seqlen 8192
+(batch 2, heads 32), synthetic seeded N(0,1) inputs resident in HBM.  Prints ONE JSON line.
+
+A step is one forward pass over the whole batch through the C ABI (fa_fwd) on torch's current stream.
+`roofline` prices the kernel against the dense fp16 MFMA peak with the algorithmic FLOPs 4*B*H*D*pairs
+(pairs = unmasked (query,key) pairs per head); its duration is measured with HIP events on that stream.
+`cpu_baseline` times the CPU oracle (a port of the reference's CPU verifier) on a bounded row sample of the
+same workload on this machine's host cores and extrapolates to the whole problem.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO)
+sys.path.insert(0, os.path.join(REPO, "tests"))
+
+PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 MFMA ("2.5 PFLOP/s")
+
+WORKLOADS = {
+    # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
+    "c1": (1, 4, 256, 64, 0, False, -1, 1.0, 0.0, 1.0, 27),
+    "c2": (4, 16, 2048, 64, 0, True, -1, 1.0, 0.0, 1.0, 28),
+    "c3": (2, 32, 8192, 128, 0, True, -1, 1.0, 0.0, 1.0, 29),
+    "c4": (1, 32, 16384, 128, 1, True, 1024, 1.0, 0.0, 1.0, 30),
+    "c5": (1, 64, 32768, 128, 0, True, -1, 0.5, 0.01, 8.0, 31),
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline sample; 0 disables")
+    ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards by (batch, head) with no "
+                 "communication, but no multi-GPU run is part of this benchmark)")
+
+    import numpy as np
+    import torch
+    from __graft_entry__ import load_package
+    from parity_util import TOL, errors, from_torch, make_inputs, sample_rows, to_torch
+
+    fa = load_package()
+    fa.lib()    # raises if the HIP library is missing: there is no fallback path
+    B, H, S, D, dtype, causal, wl, sigma, frac, mult, seed = WORKLOADS[args.workload]
+    shape = (B, H, S, D)
+    q, k, v = make_inputs(fa, shape, dtype, seed, sigma, frac, mult)
+    tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    out = torch.empty_like(tq)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+
+    def step():
+        fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, out=out, lse=lse)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(args.steps):
+        step()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]
+    avg_kernel_ms = float(np.mean(kernel_ms))
+
+    flops = fa.lib().fa_algorithmic_flops(B, H, S, D, int(causal), wl, -1)
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    kernel_tflops = flops / (avg_kernel_ms * 1e-3) / 1e12
+    algo_bytes = 4 * B * H * S * D * 2 + B * H * S * 4
+
+    result = {
+        "metric": "attn fwd TFLOPS + % of fp16 MFMA peak, hd128 causal seq 8192, 1 GPU",
+        "value": round(tflops, 2), "unit": "TFLOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D} "
+                               f"{'causal' if causal else 'non-causal'}{f' window_left {wl}' if wl >= 0 else ''}, "
+                               f"scale 1/sqrt({D}), fp32 accumulate, O + logsumexp",
+                   "seed": seed, "sigma": sigma, "algorithmic_flops": flops, "algorithmic_bytes": algo_bytes},
+        "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
+    }
+
+    if args.check_rows > 0:
+        import oracle_binding as ob
+        rows = sample_rows(shape, args.check_rows, seed)
+        o_ref, lse_ref = ob.rows(q, k, v, rows, dtype, None, causal, wl, -1)
+        err = errors(ob.to_f32(from_torch(out), dtype).reshape(-1, D)[rows], ob.to_f32(o_ref, dtype),
+                     lse.cpu().numpy().reshape(-1)[rows], lse_ref)
+        err["rows_checked"] = int(len(rows))
+        err["within_tolerance"] = bool(err["nonfinite"] == 0 and err["max_abs"] <= TOL[dtype]["max_abs"]
+                                       and err["rel_l2"] <= TOL[dtype]["rel_l2"] and err["lse_abs"] <= TOL[dtype]["lse_abs"])
+        result["parity"] = err
+
+    if args.cpu_seconds > 0:
+        import oracle_binding as ob
+        cores = ob.default_threads()
+        rng = np.random.default_rng(seed)
+        probe = np.sort(rng.integers(0, B * H * S, size=64))
+        t = time.perf_counter()
+        ob.rows(q, k, v, probe, dtype, None, causal, wl, -1, threads=cores)
+        per_row = max((time.perf_counter() - t) / len(probe), 1e-6)
+        n = int(min(B * H * S, max(256, args.cpu_seconds / per_row)))
+        sample = np.sort(rng.choice(B * H * S, size=n, replace=False))
+        t = time.perf_counter()
+        ob.rows(q, k, v, sample, dtype, None, causal, wl, -1, threads=cores)
+        dt = time.perf_counter() - t
+        pairs = 0
+        for r in sample.tolist():
+            i = r % S
+            lo = max(0, i - wl) if wl >= 0 else 0
+            hi = i if causal else S - 1
+            pairs += hi - lo + 1
+        cpu_tflops = 4.0 * D * pairs / dt / 1e12
+        result["cpu_baseline"] = {
+            "value": round(cpu_tflops, 5), "unit": "TFLOPS", "cores": cores, "kind": "port",
+            "sample": f"{n} uniformly sampled query rows of the same workload ({pairs} unmasked pairs), "
+                      f"{dt:.1f} s on {cores} threads; extrapolated whole problem: {flops / (cpu_tflops * 1e12):.0f} s",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

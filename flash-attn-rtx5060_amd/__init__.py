@@ -1,0 +1,189 @@
+"""Python binding of libfa_fwd_gfx950.so (ctypes over the C ABI in include/fa_fwd.h).
+
+Mirrors the reference operator ``run_flash_attention``
+(reference src/flash_forward.h:593-612) for callers that hold their tensors in
+PyTorch: same argument meaning, tensors are contiguous [B, N, S, d] fp16/bf16 on
+the GPU.  PyTorch is used only for device memory and the current stream; all
+arithmetic happens in the HIP library.  There is no fallback: if the shared
+library has not been built, importing a symbol from it raises.
+
+The directory name contains a hyphen, so the package is loaded by path::
+
+    import importlib.util, sys
+    spec = importlib.util.spec_from_file_location(
+        "flash_attn_rtx5060_amd", "<repo>/flash-attn-rtx5060_amd/__init__.py")
+    mod = importlib.util.module_from_spec(spec); sys.modules[spec.name] = mod
+    spec.loader.exec_module(mod)
+"""
+import ctypes
+import math
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfa_fwd_gfx950.so")
+HOST_LIB_PATH = os.path.join(_HERE, "lib", "libfa_host.so")
+HARNESS_PATH = os.path.join(_HERE, "bin", "fa_harness")
+
+FA_OK = 0
+FA_ERR_NULL_POINTER = -1
+FA_ERR_BAD_SHAPE = -2
+FA_ERR_HEAD_DIM = -3
+FA_ERR_SEQLEN_MULTIPLE = -4
+FA_ERR_UNSUPPORTED = -5
+FA_ERR_DTYPE = -6
+FA_ERR_SCALE = -7
+FA_ERR_DEVICE = -8
+FA_ERR_NO_DEVICE = -9
+FA_ERR_TOO_LARGE = -10
+FA_DTYPE_F16 = 0
+FA_DTYPE_BF16 = 1
+FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT = 0, 1, 2
+FA_TILE_SKIP, FA_TILE_PARTIAL, FA_TILE_FULL = 0, 1, 2
+
+#: every symbol include/fa_fwd.h declares
+EXPORTED_SYMBOLS = (
+    "fa_fwd_validate", "fa_fwd", "run_flash_attention", "fa_strerror", "fa_last_device_error",
+    "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
+    "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
+    "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
+    "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
+    "fa_event_elapsed_ms", "fa_event_destroy",
+)
+
+
+class FaFwdParams(ctypes.Structure):
+    """struct fa_fwd_params of include/fa_fwd.h (field-for-field)."""
+    _fields_ = [
+        ("Q", ctypes.c_void_p), ("K", ctypes.c_void_p), ("V", ctypes.c_void_p), ("O", ctypes.c_void_p),
+        ("L", ctypes.c_void_p), ("M", ctypes.c_void_p),
+        ("B", ctypes.c_int), ("N", ctypes.c_int), ("S", ctypes.c_int), ("d", ctypes.c_int),
+        ("Tr", ctypes.c_int), ("Tc", ctypes.c_int),
+        ("softmax_scale", ctypes.c_float), ("dropout_prob", ctypes.c_float),
+        ("seed", ctypes.c_ulonglong), ("states", ctypes.c_void_p),
+        ("window_size_left", ctypes.c_int), ("window_size_right", ctypes.c_int),
+        ("alibi_slopes_ptr", ctypes.c_void_p), ("split_num", ctypes.c_int),
+        ("dtype", ctypes.c_int), ("is_causal", ctypes.c_int), ("sched", ctypes.c_int),
+    ]
+
+
+class FaError(RuntimeError):
+    def __init__(self, status, detail=""):
+        self.status = status
+        msg = lib().fa_strerror(status).decode()
+        super().__init__(f"fa_fwd status {status}: {msg}{(' (' + detail + ')') if detail else ''}")
+
+
+_lib = None
+_host = None
+
+
+def lib():
+    """The C-ABI library; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `make -C {_HERE}` (hipcc, gfx950) first")
+        L = ctypes.CDLL(LIB_PATH)
+        L.fa_strerror.restype = ctypes.c_char_p
+        L.fa_strerror.argtypes = [ctypes.c_int]
+        L.fa_last_device_error.restype = ctypes.c_char_p
+        L.fa_fwd_validate.argtypes = [ctypes.POINTER(FaFwdParams)]
+        L.fa_fwd.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
+        L.run_flash_attention.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6 + [ctypes.c_int] * 5 + [
+            ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+        L.fa_sched_num_items.restype = ctypes.c_longlong
+        L.fa_sched_num_items.argtypes = [ctypes.c_int] * 4
+        L.fa_sched_item.argtypes = [ctypes.c_int] * 7 + [ctypes.c_longlong, ctypes.POINTER(ctypes.c_int),
+                                                         ctypes.POINTER(ctypes.c_int)]
+        L.fa_sched_tile_range.restype = None
+        L.fa_sched_tile_range.argtypes = [ctypes.c_int] * 7 + [ctypes.POINTER(ctypes.c_int)] * 2
+        L.fa_sched_classify.argtypes = [ctypes.c_int] * 7
+        L.fa_count_pairs.restype = ctypes.c_longlong
+        L.fa_count_pairs.argtypes = [ctypes.c_int] * 4
+        L.fa_algorithmic_flops.restype = ctypes.c_double
+        L.fa_algorithmic_flops.argtypes = [ctypes.c_int] * 7
+        _lib = L
+    return _lib
+
+
+def host_lib():
+    """Host-side helper library (seeded input generator, host/fa_inputs.h)."""
+    global _host
+    if _host is None:
+        if not os.path.exists(HOST_LIB_PATH):
+            raise RuntimeError(f"{HOST_LIB_PATH} is missing: run `make -C {_HERE}` first")
+        H = ctypes.CDLL(HOST_LIB_PATH)
+        H.fa_fill_normal.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int, ctypes.c_int, ctypes.c_uint64,
+                                     ctypes.c_uint32, ctypes.c_float, ctypes.c_double, ctypes.c_float, ctypes.c_int]
+        H.fa_input_normal.restype = ctypes.c_float
+        H.fa_input_normal.argtypes = [ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint64]
+        H.fa_input_row_selected.argtypes = [ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_double]
+        H.fa_philox4x32_10.restype = None
+        H.fa_philox4x32_10.argtypes = [ctypes.POINTER(ctypes.c_uint32)] * 3
+        for name, rt, at in (("fa_f32_to_f16_bits", ctypes.c_uint16, ctypes.c_float),
+                             ("fa_f32_to_bf16_bits", ctypes.c_uint16, ctypes.c_float),
+                             ("fa_f16_bits_to_f32", ctypes.c_float, ctypes.c_uint16),
+                             ("fa_bf16_bits_to_f32", ctypes.c_float, ctypes.c_uint16)):
+            getattr(H, name).restype = rt
+            getattr(H, name).argtypes = [at]
+        _host = H
+    return _host
+
+
+def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
+                window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO):
+    p = FaFwdParams()
+    p.Q, p.K, p.V, p.O, p.L = q_ptr or None, k_ptr or None, v_ptr or None, o_ptr or None, lse_ptr or None
+    p.B, p.N, p.S, p.d = B, N, S, d
+    p.softmax_scale = (1.0 / math.sqrt(d)) if softmax_scale is None else softmax_scale
+    p.window_size_left, p.window_size_right = window_left, window_right
+    p.dtype, p.is_causal, p.sched = dtype, int(bool(causal)), sched
+    return p
+
+
+def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
+                            return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO):
+    """O, LSE = attention(q, k, v) on the GPU through fa_fwd(); torch tensors [B, N, S, d]."""
+    import torch
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise ValueError("q, k, v must live on the GPU")
+    if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k, v must share dtype float16 or bfloat16")
+    if q.shape != k.shape or q.shape != v.shape or q.dim() != 4:
+        raise ValueError("q, k, v must share shape [B, N, S, d]")
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        raise ValueError("q, k, v must be contiguous [B, N, S, d]")
+    B, N, S, d = q.shape
+    if out is None:
+        out = torch.empty_like(q)
+    if return_lse and lse is None:
+        lse = torch.empty((B, N, S), dtype=torch.float32, device=q.device)
+    p = make_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                    lse.data_ptr() if return_lse else 0, softmax_scale, causal, window_left, window_right,
+                    FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched)
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
+    if st != FA_OK:
+        raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
+    return (out, lse) if return_lse else out
+
+
+def run_flash_attention(B, N, S, d, Q, K, V, O, L=None, M=None, Is_dropout=False, Is_causal=False, Is_local=False,
+                        Has_alibi=False, window_size=0, alibi_slopes=None, dropout_prob=0.0, states=None):
+    """The reference's entry point with its argument order (flash_forward.h:593-612); Q..L are torch
+    tensors (or None) whose device pointers are passed through; returns the status code."""
+    def ptr(t):
+        return None if t is None else ctypes.c_void_p(t.data_ptr())
+    return lib().run_flash_attention(B, N, S, d, ptr(Q), ptr(K), ptr(V), ptr(O), ptr(L), ptr(M), int(Is_dropout),
+                                     int(Is_causal), int(Is_local), int(Has_alibi), int(window_size),
+                                     ptr(alibi_slopes), float(dropout_prob), ptr(states))
+
+
+def fill_normal(rows, d, dtype, seed, tensor, sigma=1.0, fraction=0.0, row_mult=1.0, nthreads=8):
+    """numpy uint16 array [rows, d] of storage bits from the harness's seeded generator."""
+    import numpy as np
+    out = np.empty((rows, d), dtype=np.uint16)
+    rc = host_lib().fa_fill_normal(out.ctypes.data, rows, d, dtype, seed, tensor, sigma, fraction, row_mult, nthreads)
+    if rc != 0:
+        raise ValueError("fa_fill_normal rejected its arguments")
+    return out

@@ -1,0 +1,228 @@
+// C ABI of the gfx950 FlashAttention forward library (see include/fa_fwd.h).
+//
+// Role of the reference's launcher run_flash_attention / run_kernel<>
+// (reference src/flash_forward.h:369-665): argument checking, derived
+// parameters, kernel selection and launch.  Unlike the reference it never
+// exits, aborts or throws, launches asynchronously on the caller's stream,
+// keeps no global descriptor state, and does not time or print.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "fa_fwd.h"
+#include "fa_kernel_args.h"
+#include "fa_sched.h"
+
+hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, long long n_items, hipStream_t stream);
+
+namespace {
+constexpr int kWavesPerGroup = 8;
+constexpr int kBlockRows = 32 * kWavesPerGroup;
+constexpr int kBlockKeysHost = 64;
+
+thread_local char g_last_error[256] = "";
+
+int device_fail(hipError_t e, const char *what)
+{
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
+    return FA_ERR_DEVICE;
+}
+}  // namespace
+
+extern "C" {
+
+const char *fa_strerror(int status)
+{
+    switch (status) {
+    case FA_OK: return "ok";
+    case FA_ERR_NULL_POINTER: return "Q, K, V or O is NULL";
+    case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
+    case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
+    case FA_ERR_SEQLEN_MULTIPLE: return "seqlen must be a multiple of 128";
+    case FA_ERR_UNSUPPORTED: return "dropout and ALiBi are not supported";
+    case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
+    case FA_ERR_SCALE: return "softmax_scale must be finite and positive";
+    case FA_ERR_DEVICE: return "HIP runtime error";
+    case FA_ERR_NO_DEVICE: return "no gfx950 device visible";
+    case FA_ERR_TOO_LARGE: return "problem too large for the kernel's index range";
+    default: return "unknown status";
+    }
+}
+
+const char *fa_last_device_error(void) { return g_last_error; }
+
+int fa_sched_block_rows(int d) { (void)d; return kBlockRows; }
+int fa_sched_block_keys(int d) { (void)d; return kBlockKeysHost; }
+
+long long fa_sched_num_items(int B, int N, int S, int d)
+{
+    const int br = fa_sched_block_rows(d);
+    return (long long)B * N * ((S + br - 1) / br);
+}
+
+int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left, int window_right,
+                  long long item, int *bh, int *q_begin)
+{
+    if (B <= 0 || N <= 0 || S <= 0 || !bh || !q_begin) return FA_ERR_BAD_SHAPE;
+    const int br = fa_sched_block_rows(d);
+    const int nqb = (S + br - 1) / br;
+    if (item < 0 || item >= (long long)B * N * nqb) return FA_ERR_BAD_SHAPE;
+    int L, R, qb;
+    fa_mask_bounds(S, is_causal, window_left, window_right, &L, &R);
+    fa_item_decode(item, B * N, nqb, (L < S || R < S) ? 1 : 0, bh, &qb);
+    *q_begin = qb * br;
+    return FA_OK;
+}
+
+void fa_sched_tile_range(int S, int block_keys, int is_causal, int window_left, int window_right,
+                         int q_begin, int rows, int *tile_lo, int *tile_hi)
+{
+    int L, R;
+    fa_mask_bounds(S, is_causal, window_left, window_right, &L, &R);
+    fa_tile_range(S, block_keys, L, R, q_begin, rows, tile_lo, tile_hi);
+}
+
+int fa_sched_classify(int block_keys, int is_causal, int window_left, int window_right,
+                      int q_begin, int rows, int tile)
+{
+    // "unbounded" only has to exceed every reachable |i-j|
+    const int big = 0x3fffffff;
+    int L = window_left < 0 ? big : window_left;
+    int R = window_right < 0 ? big : window_right;
+    if (is_causal) R = 0;
+    return fa_tile_class(block_keys, L, R, q_begin, rows, tile);
+}
+
+long long fa_count_pairs(int S, int is_causal, int window_left, int window_right)
+{
+    int L, R;
+    fa_mask_bounds(S, is_causal, window_left, window_right, &L, &R);
+    long long pairs = 0;
+    for (int i = 0; i < S; ++i) {
+        int lo = i - L < 0 ? 0 : i - L;
+        int hi = i + R > S - 1 ? S - 1 : i + R;
+        pairs += hi - lo + 1;
+    }
+    return pairs;
+}
+
+double fa_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
+{
+    return 4.0 * (double)B * (double)N * (double)d * (double)fa_count_pairs(S, is_causal, window_left, window_right);
+}
+
+int fa_fwd_validate(const fa_fwd_params *p)
+{
+    if (!p || !p->Q || !p->K || !p->V || !p->O) return FA_ERR_NULL_POINTER;
+    if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
+    if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
+    if (p->S % 128 != 0) return FA_ERR_SEQLEN_MULTIPLE;
+    if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
+    if (p->dropout_prob != 0.0f || p->states != nullptr || p->alibi_slopes_ptr != nullptr) return FA_ERR_UNSUPPORTED;
+    if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
+    const long long bh = (long long)p->B * p->N;
+    if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    return FA_OK;
+}
+
+int fa_fwd(const fa_fwd_params *p, void *stream)
+{
+    const int st = fa_fwd_validate(p);
+    if (st != FA_OK) return st;
+
+    FaKernelArgs a;
+    a.Q = static_cast<const uint16_t *>(p->Q);
+    a.K = static_cast<const uint16_t *>(p->K);
+    a.V = static_cast<const uint16_t *>(p->V);
+    a.O = static_cast<uint16_t *>(p->O);
+    a.lse = p->L;
+    a.BH = p->B * p->N;
+    a.S = p->S;
+    a.n_qblocks = (p->S + kBlockRows - 1) / kBlockRows;
+    fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
+    const int masked = (a.L < p->S || a.R < p->S) ? 1 : 0;
+    a.descending = masked;
+    a.scale = p->softmax_scale;
+    a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
+
+    const long long n_items = (long long)a.BH * a.n_qblocks;
+    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, n_items, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return device_fail(e, "forward launch");
+    return FA_OK;
+}
+
+int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, void *O, void *L, void *M,
+                        int Is_dropout, int Is_causal, int Is_local, int Has_alibi, int window_size,
+                        float *alibi_slopes, float dropout_prob, void *states)
+{
+    (void)M;
+    (void)states;
+    (void)alibi_slopes;
+    if (Is_dropout || Has_alibi) return FA_ERR_UNSUPPORTED;
+    if (d <= 0) return FA_ERR_HEAD_DIM;
+    fa_fwd_params p;
+    memset(&p, 0, sizeof(p));
+    p.Q = Q; p.K = K; p.V = V; p.O = O;
+    p.L = static_cast<float *>(L);
+    p.B = B; p.N = N; p.S = S; p.d = d;
+    p.softmax_scale = (float)(1.0 / sqrt((double)d));      // flash_forward.h:639
+    p.dropout_prob = dropout_prob;
+    p.window_size_left = Is_local ? window_size : -1;      // flash_forward.h:640-641, mask.h:55
+    p.window_size_right = Is_local ? window_size : -1;
+    if (Is_local && window_size < 0) { p.window_size_left = p.window_size_right = 0; }
+    p.dtype = FA_DTYPE_F16;
+    p.is_causal = Is_causal ? 1 : 0;
+    const int st = fa_fwd(&p, nullptr);
+    if (st != FA_OK) return st;
+    hipError_t e = hipStreamSynchronize(nullptr);           // flash_forward.h:655
+    if (e != hipSuccess) return device_fail(e, "synchronize");
+    return FA_OK;
+}
+
+/* ---------------- thin device layer ---------------- */
+int fa_dev_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int fa_dev_name(char *buf, size_t len, int *compute_units, int *clock_khz)
+{
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, 0);
+    if (e != hipSuccess) return device_fail(e, "hipGetDeviceProperties");
+    if (buf && len) { snprintf(buf, len, "%s (%s)", prop.name, prop.gcnArchName); }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    return FA_OK;
+}
+
+#define FA_DEV(call, what) do { hipError_t e_ = (call); if (e_ != hipSuccess) return device_fail(e_, what); } while (0)
+
+int fa_dev_malloc(void **ptr, size_t bytes) { if (!ptr) return FA_ERR_NULL_POINTER; FA_DEV(hipMalloc(ptr, bytes), "hipMalloc"); return FA_OK; }
+int fa_dev_free(void *ptr) { FA_DEV(hipFree(ptr), "hipFree"); return FA_OK; }
+int fa_dev_h2d(void *dst, const void *src, size_t bytes) { FA_DEV(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy H2D"); return FA_OK; }
+int fa_dev_d2h(void *dst, const void *src, size_t bytes) { FA_DEV(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), "hipMemcpy D2H"); return FA_OK; }
+int fa_dev_memset(void *dst, int value, size_t bytes) { FA_DEV(hipMemset(dst, value, bytes), "hipMemset"); return FA_OK; }
+int fa_dev_sync(void) { FA_DEV(hipDeviceSynchronize(), "hipDeviceSynchronize"); return FA_OK; }
+int fa_event_create(void **ev)
+{
+    if (!ev) return FA_ERR_NULL_POINTER;
+    hipEvent_t e;
+    FA_DEV(hipEventCreate(&e), "hipEventCreate");
+    *ev = e;
+    return FA_OK;
+}
+int fa_event_record(void *ev, void *stream) { FA_DEV(hipEventRecord(static_cast<hipEvent_t>(ev), static_cast<hipStream_t>(stream)), "hipEventRecord"); return FA_OK; }
+int fa_event_sync(void *ev) { FA_DEV(hipEventSynchronize(static_cast<hipEvent_t>(ev)), "hipEventSynchronize"); return FA_OK; }
+int fa_event_elapsed_ms(void *start, void *stop, float *ms)
+{
+    if (!ms) return FA_ERR_NULL_POINTER;
+    FA_DEV(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)), "hipEventElapsedTime");
+    return FA_OK;
+}
+int fa_event_destroy(void *ev) { FA_DEV(hipEventDestroy(static_cast<hipEvent_t>(ev)), "hipEventDestroy"); return FA_OK; }
+
+}  // extern "C"

@@ -1,0 +1,25 @@
+// Kernel argument block of the gfx950 forward kernel.
+// Plays the part of the reference's mykernelParamType (reference
+// include/utils.h:143-165) on the device side: pointers, sizes, the folded
+// softmax scale and the effective mask bounds.
+#ifndef FA_KERNEL_ARGS_H
+#define FA_KERNEL_ARGS_H
+#include <stdint.h>
+
+struct FaKernelArgs {
+    const uint16_t *Q;
+    const uint16_t *K;
+    const uint16_t *V;
+    uint16_t *O;
+    float *lse;          // may be null
+    int BH;              // batch * heads
+    int S;
+    int n_qblocks;       // query blocks per head
+    int descending;      // 1: item rank 0 is the last query block (longest first)
+    int L;               // key j visible to query i iff i - L <= j <= i + R
+    int R;
+    float scale;         // softmax scale
+    float scale_log2e;   // softmax scale * log2(e)
+};
+
+#endif

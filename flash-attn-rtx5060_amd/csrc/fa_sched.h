@@ -1,0 +1,63 @@
+// Tile scheduler arithmetic shared by the gfx950 kernel and its host mirror.
+//
+// Replaces the reference's in-kernel Schedule<0,...>::next
+// (reference src/flash_forward.h:43-64): the same key-tile clipping for causal
+// and local masks, but with one-sided windows, a longest-first work order and
+// a per-tile classification so that element masks are applied only where a
+// tile straddles a mask edge and fully masked tiles are never visited
+// (the reference masks every tile, src/mask.h:10-84).
+#ifndef FA_SCHED_H
+#define FA_SCHED_H
+
+#if defined(__HIPCC__)
+#define FA_HD __host__ __device__ __forceinline__
+#else
+#define FA_HD static inline
+#endif
+
+// Effective mask bounds: key j is visible to query i iff  i - L <= j <= i + R.
+// `S` stands in for "unbounded" (no |i-j| can reach it).
+FA_HD void fa_mask_bounds(int S, int is_causal, int window_left, int window_right, int *L, int *R)
+{
+    int r = (window_right < 0 || window_right > S) ? S : window_right;
+    int l = (window_left < 0 || window_left > S) ? S : window_left;
+    if (is_causal) r = 0;
+    *L = l;
+    *R = r;
+}
+
+// Inclusive key-tile range visited by query rows [q_begin, q_begin + rows).
+FA_HD void fa_tile_range(int S, int block_keys, int L, int R, int q_begin, int rows, int *tile_lo, int *tile_hi)
+{
+    int lo_key = q_begin - L;
+    if (lo_key < 0) lo_key = 0;
+    int hi_key = q_begin + rows - 1 + R;
+    if (hi_key > S - 1) hi_key = S - 1;
+    *tile_lo = lo_key / block_keys;
+    *tile_hi = hi_key / block_keys;
+}
+
+// 0 = every (query,key) pair masked, 2 = none masked, 1 = mixed.
+FA_HD int fa_tile_class(int block_keys, int L, int R, int q_begin, int rows, int tile)
+{
+    const int k0 = tile * block_keys, k1 = k0 + block_keys - 1;
+    const int qa = q_begin, qb = q_begin + rows - 1;
+    if (k0 > qb + R || k1 < qa - L) return 0;
+    if (k1 <= qa + R && k0 >= qb - L) return 2;
+    return 1;
+}
+
+// Work item `item` (0 is dispatched first) -> (batch*heads + head, query block).
+// Items are ordered by decreasing number of key tiles: with a causal or
+// left-window mask the tile count grows with the query block index, so the
+// last query block of every head goes first.  Heads vary fastest so that
+// consecutively dispatched workgroups, which the hardware deals round-robin
+// over the eight XCDs, keep head (bh % 8) on one XCD's L2 when B*N % 8 == 0.
+FA_HD void fa_item_decode(long long item, int BH, int n_qblocks, int descending, int *bh, int *qblock)
+{
+    const int rank = (int)(item / BH);
+    *bh = (int)(item % BH);
+    *qblock = descending ? (n_qblocks - 1 - rank) : rank;
+}
+
+#endif

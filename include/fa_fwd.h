@@ -1,0 +1,163 @@
+/*
+ * C ABI of the MI355X (gfx950) FlashAttention forward library, libfa_fwd_gfx950.so.
+ *
+ * Drop-in boundary for the reference operator `run_flash_attention`
+ * (reference src/flash_forward.h:593-665) and its kernel argument block
+ * `mykernelParamType` (reference include/utils.h:143-165).  Plain C types
+ * only: device pointers are `void *`, booleans are `int`, the stream is an
+ * opaque `void *` (a hipStream_t, NULL = the default stream).
+ *
+ * Tensors are contiguous [B, N, S, d] 16-bit (fp16 or bf16), exactly as the
+ * reference lays them out (reference src/main.cu:182, flash_forward.h:378-381);
+ * the logsumexp output is fp32 [B, N, S].
+ */
+#ifndef FA_FWD_H
+#define FA_FWD_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  The reference exits, aborts, asserts or throws instead
+ * (include/utils.h:16-23, flash_forward.h:384-387,587-589); nothing here
+ * does: every entry point returns one of these. */
+enum {
+    FA_OK = 0,
+    FA_ERR_NULL_POINTER = -1,      /* Q, K, V or O is NULL                                  */
+    FA_ERR_BAD_SHAPE = -2,         /* B, N or S is not positive                              */
+    FA_ERR_HEAD_DIM = -3,          /* d not in {64, 128}: reference throws, flash_forward.h:587 */
+    FA_ERR_SEQLEN_MULTIPLE = -4,   /* S % 128 != 0: reference assumes it silently, :134,637  */
+    FA_ERR_UNSUPPORTED = -5,       /* dropout or ALiBi requested                             */
+    FA_ERR_DTYPE = -6,             /* dtype is neither FA_DTYPE_F16 nor FA_DTYPE_BF16        */
+    FA_ERR_SCALE = -7,             /* softmax_scale is not a finite positive number          */
+    FA_ERR_DEVICE = -8,            /* a HIP runtime call failed; see fa_last_device_error()  */
+    FA_ERR_NO_DEVICE = -9,         /* no gfx950 device is visible                            */
+    FA_ERR_TOO_LARGE = -10         /* B*N*S*d or the work-item count overflows the kernel's index range */
+};
+
+enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
+
+/* How work items (batch, head, query block) reach the compute units. */
+enum {
+    FA_SCHED_AUTO = 0,        /* the library picks                                            */
+    FA_SCHED_DISPATCH = 1,    /* one workgroup per work item, launched longest-first          */
+    FA_SCHED_PERSISTENT = 2   /* one workgroup per CU walks the longest-first list            */
+};
+
+/*
+ * Argument block.  The first twenty fields are those of the reference's
+ * mykernelParamType (include/utils.h:143-165) in the same order with the same
+ * meaning; the fields after `split_num` are what the reference passes as
+ * template booleans (flash_forward.h:369) or hard-wires.
+ */
+typedef struct fa_fwd_params {
+    const void *Q;            /* [B,N,S,d] device                                             */
+    const void *K;
+    const void *V;
+    void *O;                  /* [B,N,S,d] device, fully overwritten                          */
+    float *L;                 /* [B,N,S] fp32 logsumexp (natural log) or NULL.  The reference
+                                 accepts L and never writes it (flash_forward.h:602,628-644). */
+    float *M;                 /* unused, as in the reference; may be NULL                     */
+    int B;
+    int N;                    /* heads                                                        */
+    int S;
+    int d;
+    int Tr;                   /* ignored on input (the reference derives them, :637-638)      */
+    int Tc;
+    float softmax_scale;      /* the reference sets 1/sqrt(d) itself, flash_forward.h:639     */
+    float dropout_prob;       /* must be 0                                                    */
+    unsigned long long seed;  /* unused                                                       */
+    void *states;             /* dropout RNG states: must be NULL                             */
+    int window_size_left;     /* keys with i - j > left are masked;  < 0 = unbounded          */
+    int window_size_right;    /* keys with j - i > right are masked; < 0 = unbounded          */
+    const float *alibi_slopes_ptr; /* must be NULL                                            */
+    int split_num;            /* unused, as in the reference (utils.h:164)                    */
+    /* --- beyond mykernelParamType --- */
+    int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                 */
+    int is_causal;            /* keys with j > i are masked (mask.h:27-38)                    */
+    int sched;                /* FA_SCHED_*                                                   */
+} fa_fwd_params;
+
+/* Checks a parameter block without touching any device.  Returns FA_OK or the
+ * first violated FA_ERR_*.  (Replaces the reference's abort/throw/assert paths.) */
+int fa_fwd_validate(const fa_fwd_params *p);
+
+/* Enqueues the forward pass on `stream` and returns without synchronising.
+ * Allocates nothing; Q/K/V are read-only, O (and L when non-NULL) are
+ * overwritten.  Re-entrant: the library keeps no per-call global state
+ * (the reference keeps four global CUtensorMaps, flash_forward.h:17-20). */
+int fa_fwd(const fa_fwd_params *p, void *stream);
+
+/*
+ * The reference's entry point, same name, argument order and meaning
+ * (flash_forward.h:593-612; its only call site is src/main.cu:99):
+ * fp16 tensors, softmax scale 1/sqrt(d), `Is_local` masks |i-j| > window_size
+ * on both sides (mask.h:55-66), `Is_causal && Is_local` is "left window, right 0".
+ * Like the reference it runs on the default stream of the current device and
+ * returns after the kernel has finished (flash_forward.h:655); unlike it, it
+ * prints nothing, returns a status, and fills L with the fp32 logsumexp when
+ * L is non-NULL.  M is ignored.  Dropout and ALiBi return FA_ERR_UNSUPPORTED.
+ */
+int run_flash_attention(int B, int N, int S, int d,
+                        void *Q, void *K, void *V, void *O,
+                        void *L, void *M,
+                        int Is_dropout, int Is_causal, int Is_local, int Has_alibi,
+                        int window_size, float *alibi_slopes,
+                        float dropout_prob, void *states);
+
+const char *fa_strerror(int status);
+/* Text of the last HIP error seen by the calling thread ("" if none). */
+const char *fa_last_device_error(void);
+
+/* ------------------------------------------------------------------ */
+/* Tile scheduler, host side.  Mirrors what the kernel computes, so the */
+/* schedule can be checked without a GPU.  Replaces Schedule<0,...>     */
+/* (flash_forward.h:22-65).                                             */
+/* ------------------------------------------------------------------ */
+enum { FA_TILE_SKIP = 0, FA_TILE_PARTIAL = 1, FA_TILE_FULL = 2 };
+
+/* Query rows per work item and keys per tile used for head dim d. */
+int fa_sched_block_rows(int d);
+int fa_sched_block_keys(int d);
+/* Number of work items for a problem: B*N*ceil(S/block_rows). */
+long long fa_sched_num_items(int B, int N, int S, int d);
+/* Work item `item` (0 = launched first) -> batch*N+head and first query row. */
+int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left,
+                  int window_right, long long item, int *bh, int *q_begin);
+/* Key-tile range [*tile_lo, *tile_hi] (inclusive) visited for query rows
+ * [q_begin, q_begin + rows).  Same clipping as flash_forward.h:52-61. */
+void fa_sched_tile_range(int S, int block_keys, int is_causal, int window_left,
+                         int window_right, int q_begin, int rows,
+                         int *tile_lo, int *tile_hi);
+/* Classification of key tile `tile` against query rows [q_begin, q_begin+rows). */
+int fa_sched_classify(int block_keys, int is_causal, int window_left, int window_right,
+                      int q_begin, int rows, int tile);
+/* Unmasked (query, key) pairs per head, and algorithmic FLOPs 4*B*N*d*pairs. */
+long long fa_count_pairs(int S, int is_causal, int window_left, int window_right);
+double fa_algorithmic_flops(int B, int N, int S, int d, int is_causal,
+                            int window_left, int window_right);
+
+/* ------------------------------------------------------------------ */
+/* Thin device layer so that a plain-C host harness needs no HIP header */
+/* (the role cudaMalloc/cudaMemcpy/cudaEvent* play in src/main.cu:61-101 */
+/* and flash_forward.h:646-662).                                        */
+/* ------------------------------------------------------------------ */
+int fa_dev_count(void);
+int fa_dev_name(char *buf, size_t len, int *compute_units, int *clock_khz);
+int fa_dev_malloc(void **ptr, size_t bytes);
+int fa_dev_free(void *ptr);
+int fa_dev_h2d(void *dst, const void *src, size_t bytes);
+int fa_dev_d2h(void *dst, const void *src, size_t bytes);
+int fa_dev_memset(void *dst, int value, size_t bytes);
+int fa_dev_sync(void);
+int fa_event_create(void **ev);
+int fa_event_record(void *ev, void *stream);
+int fa_event_sync(void *ev);
+int fa_event_elapsed_ms(void *start, void *stop, float *ms);
+int fa_event_destroy(void *ev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

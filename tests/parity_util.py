@@ -1,0 +1,64 @@
+"""Shared helpers of the GPU parity tests: seeded inputs, error metrics, stated tolerances."""
+import numpy as np
+
+# Stated tolerances against the CPU oracle on the same seeded inputs.
+# max-abs is the bound the task states (about one output ulp at |O| in [2,4));
+# rel-L2 and the logsumexp bound are this build's own stated bounds.
+TOL = {
+    0: dict(max_abs=2e-3, rel_l2=1e-3, lse_abs=2e-3),     # fp16
+    1: dict(max_abs=1.6e-2, rel_l2=8e-3, lse_abs=8e-3),   # bf16 (the oracle rounds every q*k product to bf16)
+}
+
+
+def make_inputs(fa, shape, dtype, seed, sigma=1.0, fraction=0.0, row_mult=1.0):
+    B, H, S, D = shape
+    rows = B * H * S
+    q = fa.fill_normal(rows, D, dtype, seed, 0, sigma, fraction, row_mult).reshape(shape)
+    k = fa.fill_normal(rows, D, dtype, seed, 1, sigma).reshape(shape)
+    v = fa.fill_normal(rows, D, dtype, seed, 2, sigma).reshape(shape)
+    return q, k, v
+
+
+def to_torch(bits, dtype, device="cuda"):
+    import torch
+    t = torch.from_numpy(bits.view(np.int16)).to(device)
+    return t.view(torch.bfloat16 if dtype == 1 else torch.float16)
+
+
+def from_torch(t):
+    import torch
+    return t.detach().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def errors(o_gpu_f32, o_ref_f32, lse_gpu=None, lse_ref=None):
+    d = o_gpu_f32.astype(np.float64) - o_ref_f32.astype(np.float64)
+    out = dict(max_abs=float(np.max(np.abs(d))) if d.size else 0.0,
+               rel_l2=float(np.sqrt(np.sum(d * d) / max(np.sum(o_ref_f32.astype(np.float64) ** 2), 1e-300))),
+               nonfinite=int(np.count_nonzero(~np.isfinite(o_gpu_f32))))
+    if lse_gpu is not None:
+        out["lse_abs"] = float(np.max(np.abs(lse_gpu.astype(np.float64) - lse_ref.astype(np.float64))))
+        out["nonfinite"] += int(np.count_nonzero(~np.isfinite(lse_gpu)))
+    return out
+
+
+def assert_within(err, dtype, what=""):
+    tol = TOL[dtype]
+    assert err["nonfinite"] == 0, f"{what}: non-finite outputs {err}"
+    assert err["max_abs"] <= tol["max_abs"], f"{what}: max-abs {err['max_abs']:.3e} > {tol['max_abs']:.1e} ({err})"
+    assert err["rel_l2"] <= tol["rel_l2"], f"{what}: rel-L2 {err['rel_l2']:.3e} > {tol['rel_l2']:.1e} ({err})"
+    if "lse_abs" in err:
+        assert err["lse_abs"] <= tol["lse_abs"], f"{what}: LSE {err['lse_abs']:.3e} > {tol['lse_abs']:.1e} ({err})"
+
+
+def sample_rows(shape, n, seed, extra=()):
+    """Seeded flat-row subset that always holds the edge rows of every head (0, 1, 31, 32, 63, 64, 127, 128,
+    255, 256, S-1 ...) plus `extra` per-head row numbers."""
+    B, H, S, D = shape
+    rng = np.random.default_rng(seed)
+    per_head = sorted({r for r in (0, 1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, S // 2, S - 2, S - 1)
+                       if 0 <= r < S} | {r for r in extra if 0 <= r < S})
+    rows = [(bh * S + r) for bh in range(B * H) for r in per_head]
+    want = max(0, n - len(rows))
+    if want:
+        rows.extend(rng.integers(0, B * H * S, size=want).tolist())
+    return np.unique(np.asarray(rows, dtype=np.int64))

@@ -1,0 +1,115 @@
+"""C-ABI boundary without a GPU: the library loads, exports every symbol include/fa_fwd.h declares, and
+rejects bad arguments with status codes (the reference exits/aborts/throws: utils.h:16-23,
+flash_forward.h:384-387,587-589)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(REPO, "include", "fa_fwd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"^\s*(?:const\s+)?(?:int|void|long long|double|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def test_header_and_library_agree(fa):
+    names = declared_functions()
+    assert sorted(fa.EXPORTED_SYMBOLS) == names
+    L = fa.lib()
+    for n in names:
+        assert getattr(L, n) is not None
+
+
+def test_struct_layout_matches_header(fa):
+    text = open(os.path.join(REPO, "include", "fa_fwd.h")).read()
+    body = re.search(r"typedef struct fa_fwd_params \{(.*?)\} fa_fwd_params;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = [re.search(r"(\w+)\s*;", line).group(1) for line in body.splitlines() if ";" in line]
+    assert fields == [f[0] for f in fa.FaFwdParams._fields_]
+    # the first twenty are mykernelParamType's, in its order (include/utils.h:143-165)
+    assert fields[:20] == ["Q", "K", "V", "O", "L", "M", "B", "N", "S", "d", "Tr", "Tc", "softmax_scale", "dropout_prob",
+                           "seed", "states", "window_size_left", "window_size_right", "alibi_slopes_ptr", "split_num"]
+
+
+def test_validate_status_codes(fa):
+    L = fa.lib()
+    ok = dict(B=2, N=8, S=2048, d=64, q_ptr=0x1000, k_ptr=0x2000, v_ptr=0x3000, o_ptr=0x4000)
+
+    def status(**kw):
+        a = dict(ok)
+        a.update(kw)
+        return L.fa_fwd_validate(ctypes.byref(fa.make_params(**a)))
+
+    def status_raw(raw, **kw):
+        a = dict(ok)
+        a.update(kw)
+        p = fa.make_params(**a)
+        for k, v in raw.items():
+            setattr(p, k, v)
+        return L.fa_fwd_validate(ctypes.byref(p))
+
+    assert status() == fa.FA_OK
+    assert L.fa_fwd_validate(None) == fa.FA_ERR_NULL_POINTER
+    for missing in ("q_ptr", "k_ptr", "v_ptr", "o_ptr"):
+        assert status(**{missing: 0}) == fa.FA_ERR_NULL_POINTER
+    assert status(B=0) == fa.FA_ERR_BAD_SHAPE
+    assert status(N=-1) == fa.FA_ERR_BAD_SHAPE
+    assert status(S=0) == fa.FA_ERR_BAD_SHAPE
+    for d in (0, 32, 96, 256):
+        assert status(d=d, softmax_scale=0.1) == fa.FA_ERR_HEAD_DIM            # the reference throws, flash_forward.h:587-589
+    for S in (64, 100, 2048 + 64):
+        assert status(S=S) == fa.FA_ERR_SEQLEN_MULTIPLE     # the reference silently assumes it
+    assert status(dtype=2) == fa.FA_ERR_DTYPE
+    assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE
+    assert status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE
+    assert status(softmax_scale=float("inf")) == fa.FA_ERR_SCALE
+    assert status_raw(dict(dropout_prob=0.1)) == fa.FA_ERR_UNSUPPORTED
+    assert status_raw(dict(states=0x10)) == fa.FA_ERR_UNSUPPORTED
+    assert status_raw(dict(alibi_slopes_ptr=0x10)) == fa.FA_ERR_UNSUPPORTED
+    assert status(B=70000, N=70000, S=128) == fa.FA_ERR_TOO_LARGE
+    # fa_fwd itself refuses the same blocks before touching any device
+    p = fa.make_params(**dict(ok, d=96))
+    assert L.fa_fwd(ctypes.byref(p), None) == fa.FA_ERR_HEAD_DIM
+
+
+def test_reference_entry_point_rejects_unsupported_flags(fa):
+    L = fa.lib()
+    args = [2, 8, 2048, 64, 0x1000, 0x2000, 0x3000, 0x4000, None, None]
+    assert L.run_flash_attention(*args, 1, 0, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_UNSUPPORTED   # dropout
+    assert L.run_flash_attention(*args, 0, 0, 0, 1, 0, None, 0.0, None) == fa.FA_ERR_UNSUPPORTED   # ALiBi
+    bad = list(args)
+    bad[3] = 48
+    assert L.run_flash_attention(*bad, 0, 0, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_HEAD_DIM
+    bad = list(args)
+    bad[4] = None
+    assert L.run_flash_attention(*bad, 0, 1, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_NULL_POINTER
+
+
+def test_strerror_covers_every_status(fa):
+    L = fa.lib()
+    seen = set()
+    for st in range(0, -11, -1):
+        msg = L.fa_strerror(st).decode()
+        assert msg and msg != "unknown status"
+        seen.add(msg)
+    assert len(seen) == 11
+    assert L.fa_strerror(-99).decode() == "unknown status"
+
+
+def test_missing_library_fails_loudly(fa, monkeypatch):
+    monkeypatch.setattr(fa, "_lib", None)
+    monkeypatch.setattr(fa, "LIB_PATH", "/nonexistent/libfa_fwd_gfx950.so")
+    with pytest.raises(RuntimeError, match="is missing"):
+        fa.lib()
+
+
+def test_python_wrapper_refuses_cpu_tensors(fa):
+    import torch
+    q = torch.zeros(1, 1, 128, 64, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        fa.flash_attention_forward(q, q, q)
