@@ -22,6 +22,7 @@ constexpr int kBlockRows = 32 * kWavesPerGroup;
 constexpr int kBlockKeysHost = 64;
 
 thread_local char g_last_error[256] = "";
+long long *g_debug_buffer = nullptr;   // set only by development builds
 
 int device_fail(hipError_t e, const char *what)
 {
@@ -145,6 +146,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.descending = masked;
     a.scale = p->softmax_scale;
     a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
+    a.dbg = g_debug_buffer;
 
     const long long n_items = (long long)a.BH * a.n_qblocks;
     hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, n_items, static_cast<hipStream_t>(stream));
@@ -179,6 +181,10 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
     if (e != hipSuccess) return device_fail(e, "synchronize");
     return FA_OK;
 }
+
+#ifdef FA_PHASE_TIMING
+void fa_debug_set_timing_buffer(long long *buf) { g_debug_buffer = buf; }
+#endif
 
 /* ---------------- thin device layer ---------------- */
 int fa_dev_count(void)

@@ -48,15 +48,29 @@ FA_HD int fa_tile_class(int block_keys, int L, int R, int q_begin, int rows, int
 }
 
 // Work item `item` (0 is dispatched first) -> (batch*heads + head, query block).
-// Items are ordered by decreasing number of key tiles: with a causal or
-// left-window mask the tile count grows with the query block index, so the
-// last query block of every head goes first.  Heads vary fastest so that
-// consecutively dispatched workgroups, which the hardware deals round-robin
-// over the eight XCDs, keep head (bh % 8) on one XCD's L2 when B*N % 8 == 0.
+//
+// Heads are taken in groups of FA_HEAD_GROUP = 8, one head per XCD: the hardware deals consecutively
+// dispatched workgroups round-robin over the eight XCDs, so with the head index fastest inside a group,
+// head (8g + x) runs on XCD x only, and the whole chip works on eight heads at a time.  One head's K and V
+// (4 MiB at seqlen 8192, head dim 128) then fit that XCD's L2 and are fetched from HBM about once instead of
+// once per query block.  Inside a group the query blocks are ordered by decreasing number of key tiles
+// (longest first): with a causal or left-window mask the tile count grows with the query block index, so
+// the last query block of every head goes first and the short ones fill the tail.
+#define FA_HEAD_GROUP 8
 FA_HD void fa_item_decode(long long item, int BH, int n_qblocks, int descending, int *bh, int *qblock)
 {
-    const int rank = (int)(item / BH);
-    *bh = (int)(item % BH);
+    const long long per_group = (long long)FA_HEAD_GROUP * n_qblocks;
+    const int full_groups = BH / FA_HEAD_GROUP;
+    int group = (int)(item / per_group);
+    int heads_here = FA_HEAD_GROUP;
+    long long rem = item - (long long)group * per_group;
+    if (group >= full_groups) {          // the last, smaller group
+        group = full_groups;
+        heads_here = BH - full_groups * FA_HEAD_GROUP;
+        rem = item - (long long)full_groups * per_group;
+    }
+    const int rank = (int)(rem / heads_here);
+    *bh = group * FA_HEAD_GROUP + (int)(rem % heads_here);
     *qblock = descending ? (n_qblocks - 1 - rank) : rank;
 }
 
