@@ -14,15 +14,22 @@
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
-hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, long long n_items, hipStream_t stream);
+hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int waves, unsigned grid, hipStream_t stream);
 
 namespace {
-constexpr int kWavesPerGroup = 8;
-constexpr int kBlockRows = 32 * kWavesPerGroup;
 constexpr int kBlockKeysHost = 64;
+constexpr int kComputeUnits = 256;      // MI355X; the persistent grid is sized from the device at run time
+
+// Workgroup shape for a problem.  The 8-wave kernel (256 query rows, one workgroup per CU) shares every K/V
+// tile among more rows; the 4-wave kernel (128 rows, two workgroups per CU) has twice as many, smaller work
+// items and wins when there are too few of the large ones to fill and balance the chip.
+int waves_for(int B, int N, int S)
+{
+    const long long big_items = (long long)B * N * ((S + 255) / 256);
+    return big_items >= 4LL * kComputeUnits ? 8 : 4;
+}
 
 thread_local char g_last_error[256] = "";
-long long *g_debug_buffer = nullptr;   // set only by development builds
 
 int device_fail(hipError_t e, const char *what)
 {
@@ -53,12 +60,12 @@ const char *fa_strerror(int status)
 
 const char *fa_last_device_error(void) { return g_last_error; }
 
-int fa_sched_block_rows(int d) { (void)d; return kBlockRows; }
+int fa_sched_block_rows(int B, int N, int S, int d) { (void)d; return 32 * waves_for(B, N, S); }
 int fa_sched_block_keys(int d) { (void)d; return kBlockKeysHost; }
 
 long long fa_sched_num_items(int B, int N, int S, int d)
 {
-    const int br = fa_sched_block_rows(d);
+    const int br = fa_sched_block_rows(B, N, S, d);
     return (long long)B * N * ((S + br - 1) / br);
 }
 
@@ -66,7 +73,7 @@ int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left, in
                   long long item, int *bh, int *q_begin)
 {
     if (B <= 0 || N <= 0 || S <= 0 || !bh || !q_begin) return FA_ERR_BAD_SHAPE;
-    const int br = fa_sched_block_rows(d);
+    const int br = fa_sched_block_rows(B, N, S, d);
     const int nqb = (S + br - 1) / br;
     if (item < 0 || item >= (long long)B * N * nqb) return FA_ERR_BAD_SHAPE;
     int L, R, qb;
@@ -140,16 +147,31 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.lse = p->L;
     a.BH = p->B * p->N;
     a.S = p->S;
-    a.n_qblocks = (p->S + kBlockRows - 1) / kBlockRows;
+    const int waves = waves_for(p->B, p->N, p->S);
+    const int block_rows = 32 * waves;
+    a.n_qblocks = (p->S + block_rows - 1) / block_rows;
     fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
     const int masked = (a.L < p->S || a.R < p->S) ? 1 : 0;
     a.descending = masked;
     a.scale = p->softmax_scale;
     a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
-    a.dbg = g_debug_buffer;
+    a.n_items = (long long)a.BH * a.n_qblocks;
 
-    const long long n_items = (long long)a.BH * a.n_qblocks;
-    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, n_items, static_cast<hipStream_t>(stream));
+    // Dispatch mode launches one workgroup per item, in list order; the hardware hands them to CUs as these
+    // free up, which is a longest-first greedy schedule.  Persistent mode launches one resident set of
+    // workgroups that walk the list themselves.
+    long long grid = a.n_items;
+    if (p->sched == FA_SCHED_PERSISTENT) {
+        int cus = kComputeUnits;
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            int n = 0;
+            if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+        }
+        const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
+        if (grid > resident) grid = resident;
+    }
+    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, waves, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
     return FA_OK;
 }
@@ -181,10 +203,6 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
     if (e != hipSuccess) return device_fail(e, "synchronize");
     return FA_OK;
 }
-
-#ifdef FA_PHASE_TIMING
-void fa_debug_set_timing_buffer(long long *buf) { g_debug_buffer = buf; }
-#endif
 
 /* ---------------- thin device layer ---------------- */
 int fa_dev_count(void)

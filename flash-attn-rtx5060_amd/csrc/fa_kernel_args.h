@@ -20,7 +20,7 @@ struct FaKernelArgs {
     int R;
     float scale;         // softmax scale
     float scale_log2e;   // softmax scale * log2(e)
-    long long *dbg;      // development timing buffer (null in production builds)
+    long long n_items;   // work items: BH * n_qblocks
 };
 
 #endif

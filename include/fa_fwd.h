@@ -40,9 +40,9 @@ enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
 
 /* How work items (batch, head, query block) reach the compute units. */
 enum {
-    FA_SCHED_AUTO = 0,        /* the library picks                                            */
+    FA_SCHED_AUTO = 0,        /* the library picks (currently FA_SCHED_DISPATCH)              */
     FA_SCHED_DISPATCH = 1,    /* one workgroup per work item, launched longest-first          */
-    FA_SCHED_PERSISTENT = 2   /* one workgroup per CU walks the longest-first list            */
+    FA_SCHED_PERSISTENT = 2   /* a resident grid sized to the CUs walks the longest-first list */
 };
 
 /*
@@ -117,8 +117,8 @@ const char *fa_last_device_error(void);
 /* ------------------------------------------------------------------ */
 enum { FA_TILE_SKIP = 0, FA_TILE_PARTIAL = 1, FA_TILE_FULL = 2 };
 
-/* Query rows per work item and keys per tile used for head dim d. */
-int fa_sched_block_rows(int d);
+/* Query rows per work item for a problem, and keys per tile for head dim d. */
+int fa_sched_block_rows(int B, int N, int S, int d);
 int fa_sched_block_keys(int d);
 /* Number of work items for a problem: B*N*ceil(S/block_rows). */
 long long fa_sched_num_items(int B, int N, int S, int d);
