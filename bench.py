@@ -19,6 +19,11 @@ sys.path.insert(0, os.path.join(REPO, "tests"))
 
 PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 MFMA ("2.5 PFLOP/s")
 
+# HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
+# worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 551.7 MB read + 136.3 MB written.
+MEASURED_HBM_BYTES = {"c3": 688.0e6}
+
 WORKLOADS = {
     # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
     "c1": (1, 4, 256, 64, 0, False, -1, 1.0, 0.0, 1.0, 27),
@@ -37,6 +42,10 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline sample; 0 disables")
     ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
+    ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2), help="0 library default, 1 dispatch, 2 persistent")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters to bytes)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards by (batch, head) with no "
@@ -57,7 +66,7 @@ def main():
     lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
 
     def step():
-        fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, out=out, lse=lse)
+        fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, out=out, lse=lse, sched=args.sched)
 
     for _ in range(args.warmup):
         step()
@@ -72,6 +81,13 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     kernel_ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]
     avg_kernel_ms = float(np.mean(kernel_ms))
+
+    if args.copy_calibration > 0:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)              # one elementwise copy kernel: reads and writes exactly this many bytes
+        torch.cuda.synchronize()
 
     flops = fa.lib().fa_algorithmic_flops(B, H, S, D, int(causal), wl, -1)
     tflops = flops / (wall_ms * 1e-3) / 1e12
@@ -89,7 +105,7 @@ def main():
                    "seed": seed, "sigma": sigma, "algorithmic_flops": flops, "algorithmic_bytes": algo_bytes},
         "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": MEASURED_HBM_BYTES.get(args.workload),
                      "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
     }
 
