@@ -83,6 +83,13 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(f"{LIB_PATH} is missing: run `make -C {_HERE}` (hipcc, gfx950) first")
+        # PyTorch ships its own copy of the HIP runtime.  A process that uses both must load PyTorch's first, so
+        # that this library binds to the same runtime instance; loaded the other way round, the second runtime
+        # to initialise reports "no ROCm-capable device".
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         L.fa_strerror.restype = ctypes.c_char_p
         L.fa_strerror.argtypes = [ctypes.c_int]
