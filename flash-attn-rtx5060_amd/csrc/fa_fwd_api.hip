@@ -14,7 +14,7 @@
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
-hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int waves, unsigned grid, hipStream_t stream);
+hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream);
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -171,7 +171,8 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
         if (grid > resident) grid = resident;
     }
-    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, waves, (unsigned)grid, static_cast<hipStream_t>(stream));
+    const int shape = waves == 8 ? 0 : 1;
+    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
     return FA_OK;
 }

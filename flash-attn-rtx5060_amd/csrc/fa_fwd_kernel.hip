@@ -201,17 +201,20 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
 }
 
 // ---------------------------------------------------------------------------
-// The kernel.  NW waves of 32 query rows each per workgroup, NST LDS stages per
-// tensor.  Every wave runs ONE instruction stream per key tile; tiles are
-// issued NST-1 iterations before their first use; one workgroup barrier per
-// tile.
+// The kernel.  NW waves per workgroup, RB blocks of 32 query rows per wave,
+// NST LDS stages per tensor.  Every wave runs ONE instruction stream per key
+// tile; tiles are issued NST-1 iterations before their first use; one
+// workgroup barrier per tile.  With RB = 2 every K/V fragment read from LDS
+// feeds two matrix instructions, and the wave needs the whole 512-entry
+// register file of its SIMD (one wave per SIMD).
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, int NW, int NST>
-__global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArgs a)
+template <bool BF16, int D, bool MASKED, int NW, int RB, int NST>
+__global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
 {
-    constexpr int BR = 32 * NW;
+    constexpr int WR = 32 * RB;                   // query rows per wave
+    constexpr int BR = WR * NW;                   // query rows per workgroup
     constexpr int CPR = D / 8;
     constexpr int ROWB = D * 2;
     constexpr int TILEB = kBlockKeys * ROWB;
@@ -219,10 +222,10 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     constexpr int IPW = INSTR / NW;               // direct-to-LDS instructions per wave per tile
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
-    constexpr int NPV = 4 * DB;                   // PV matrix instructions per tile
-    constexpr int NQK = 2 * KS;                   // QK matrix instructions per tile
-    constexpr int NM = NPV + NQK;
-    constexpr int PD = 6;                         // LDS reads run this many matrix instructions ahead
+    constexpr int NPV = 4 * DB;                   // V^T fragments per tile: (16-key slice, head-dim block)
+    constexpr int NQK = 2 * KS;                   // K fragments per tile: (head-dim slice, 32-key block)
+    constexpr int NF = NPV + NQK;                 // every fragment feeds RB matrix instructions
+    constexpr int PD = RB == 1 ? 6 : 3;           // LDS reads run this many fragments ahead
     constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
     constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
     static_assert(INSTR % NW == 0, "tile must divide over the waves");
@@ -252,26 +255,26 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     uint16_t *Oh = a.O + head_off;
 
     const int q0 = qblock * BR;
-    const int qw = q0 + wave * 32;
-    const int my_q = qw + l32;
-    const bool wave_live = qw < S;
+    const int qw = q0 + wave * WR;          // first query row of this wave
+    const int my_q = qw + l32;              // query row of row block 0 on this lane; block b adds 32*b
+    const bool wave_live = qw < S;          // S is a multiple of 128: a live wave has all its rows
 
-    u32x4 qf[KS];
-    if (wave_live) {
+    // Q^T fragments: B operand, lane = (query l32, head-dim slice 8*half..+7 of each 16)
+    u32x4 qf[RB][KS];
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-            qf[s] = *reinterpret_cast<const u32x4 *>(Qh + (size_t)my_q * D + 16 * s + 8 * half);
-    } else {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) qf[s] = u32x4{0, 0, 0, 0};
-    }
+            qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(Qh + (size_t)(my_q + 32 * b) * D + 16 * s + 8 * half)
+                                 : u32x4{0, 0, 0, 0};
 
     const int rows_in_block = S - q0 < BR ? S - q0 : BR;
     int t0, t1;                 // key tiles visited by the workgroup
     fa_tile_range(S, kBlockKeys, a.L, a.R, q0, rows_in_block, &t0, &t1);
     int my_lo = 1, my_hi = 0;   // key tiles with at least one visible pair for this wave (contiguous)
-    if (wave_live) fa_tile_range(S, kBlockKeys, a.L, a.R, qw, 32, &my_lo, &my_hi);
+    if (wave_live) fa_tile_range(S, kBlockKeys, a.L, a.R, qw, WR, &my_lo, &my_hi);
 
+    // per-lane LDS read addresses for stage 0; stage, key block and key slice are immediates
     uint32_t koff[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s)
@@ -286,6 +289,8 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
             voff[db] = lds0 + LDS_V + (uint32_t)(row0 * ROWB + ((c ^ v_swz<CPR>(row0)) << 4) + ((c4 & 1) << 3));
         }
     }
+    // direct global -> LDS tile loads: wave w issues instructions w, w+NW, ... of the tile; instruction n
+    // fills LDS bytes [n*1024, n*1024+1024) linearly, lane l supplying the swizzled source chunk.
     uint32_t gk[IPW], gv[IPW];
 #pragma unroll
     for (int i = 0; i < IPW; ++i) {
@@ -304,16 +309,20 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         for (int i = 0; i < IPW; ++i) dma_16(src, gv[i], lds0 + LDS_V + stage * TILEB + (i * NW + wave) * 1024);
     };
 
-    f32x16 o[DB];
+    f32x16 o[RB][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int b = 0; b < RB; ++b)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[db][r] = 0.0f;
-    float m_run = -INFINITY, l_a = 0.0f, l_b = 0.0f;
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][db][r] = 0.0f;
+    float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
+#pragma unroll
+    for (int b = 0; b < RB; ++b) { m_run[b] = -INFINITY; l_a[b] = 0.0f; l_b[b] = 0.0f; }
     const float c = a.scale_log2e;
     const float thresh = kRescaleLog2 / c;
-    uint32_t pk[16];            // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
-    f32x16 s0, s1;              // S^T of the tile whose softmax comes next
+    uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
+    f32x16 sx[RB][2];           // S^T of the tile whose softmax comes next: [key block 0 / 1]
 
     auto read_v = [&](uint32_t vs, int n) __attribute__((always_inline)) {
         const int t2 = n / DB, db = n % DB;
@@ -327,33 +336,46 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     auto apply_mask = [&](int tile) __attribute__((always_inline)) {
         const int kb0 = tile * kBlockKeys + 4 * half;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
-            const int j1 = j0 + 32;
-            if (j0 > my_q + a.R || j0 < my_q - a.L) s0[r] = -INFINITY;
-            if (j1 > my_q + a.R || j1 < my_q - a.L) s1[r] = -INFINITY;
+        for (int b = 0; b < RB; ++b) {
+            const int q = my_q + 32 * b;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
+                const int j1 = j0 + 32;
+                if (j0 > q + a.R || j0 < q - a.L) sx[b][0][r] = -INFINITY;
+                if (j1 > q + a.R || j1 < q - a.L) sx[b][1][r] = -INFINITY;
+            }
         }
     };
-    // row maximum of S(tile) and the decision to move the reference point; returns the factor by which
-    // everything accumulated so far has to be multiplied (1 when the reference point stays)
-    auto new_reference = [&](float mx, bool &moved) __attribute__((always_inline)) {
+    auto row_max = [&](int b) __attribute__((always_inline)) {
+        float mx = fmaxf(sx[b][0][0], sx[b][1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, sx[b][0][r]), sx[b][1][r]);
+        return fmaxf(mx, swap_halves(mx));
+    };
+    // the decision to move the reference point of row block b; returns the factor by which everything
+    // accumulated so far has to be multiplied (1 when the reference point stays)
+    auto new_reference = [&](int b, float mx, bool &moved) __attribute__((always_inline)) {
         float alpha = 1.0f;
-        const bool grow = mx > m_run + thresh;      // -inf + thresh = -inf: a first finite max always grows
+        const bool grow = mx > m_run[b] + thresh;   // -inf + thresh = -inf: a first finite max always grows
         moved = __builtin_amdgcn_ballot_w64(grow) != 0;
         if (moved) {
-            const float m_new = grow ? mx : m_run;
-            alpha = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
-            l_a *= alpha;
-            l_b *= alpha;
-            m_run = m_new;
+            const float m_new = grow ? mx : m_run[b];
+            alpha = (m_run[b] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run[b] - m_new) * c);
+            l_a[b] *= alpha;
+            l_b[b] *= alpha;
+            m_run[b] = m_new;
         }
         return alpha;
     };
-    auto scale_o = [&](float alpha) __attribute__((always_inline)) {
+    auto scale_o = [&](int b, float alpha) __attribute__((always_inline)) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+            for (int r = 0; r < 16; ++r) o[b][db][r] *= alpha;
+    };
+    auto p_operand = [&](int b, int t2) __attribute__((always_inline)) {
+        return u32x4{pk[b][4 * t2], pk[b][4 * t2 + 1], pk[b][4 * t2 + 2], pk[b][4 * t2 + 3]};
     };
 
     // ---- plain (not interleaved) pieces, used while the pipeline fills and drains
@@ -369,8 +391,8 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         for (int n = 0; n < NPV; ++n) {
             if (n + 2 < NPV) fr[n + 2] = read_v(vs, n + 2);
             const int t2 = n / DB, db = n % DB;
-            const u32x4 pb = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
-            o[db] = N::mfma(fr[n], pb, o[db]);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) o[b][db] = N::mfma(fr[n], p_operand(b, t2), o[b][db]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -380,35 +402,36 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         fr[0] = read_k(ks, 0);
         fr[1] = read_k(ks, 1);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; }
+        for (int b = 0; b < RB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sx[b][0][r] = 0.0f; sx[b][1][r] = 0.0f; }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < NQK; ++n) {
             if (n + 2 < NQK) fr[n + 2] = read_k(ks, n + 2);
-            if (n & 1) s1 = N::mfma(fr[n], qf[n >> 1], s1);
-            else s0 = N::mfma(fr[n], qf[n >> 1], s0);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) sx[b][n & 1] = N::mfma(fr[n], qf[b][n >> 1], sx[b][n & 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
-        if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, 32, tile) == 1) apply_mask(tile);
-        float mx = fmaxf(s0[0], s1[0]);
+        if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile) == 1) apply_mask(tile);
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, s0[r]), s1[r]);
-        mx = fmaxf(mx, swap_halves(mx));
-        bool moved;
-        const float alpha = new_reference(mx, moved);
-        if (moved) scale_o(alpha);
-        const float mc = (m_run == -INFINITY) ? 0.0f : m_run * c;
+        for (int b = 0; b < RB; ++b) {
+            bool moved;
+            const float alpha = new_reference(b, row_max(b), moved);
+            if (moved) scale_o(b, alpha);
+            const float mc = (m_run[b] == -INFINITY) ? 0.0f : m_run[b] * c;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[2 * i], c, -mc));
-            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[2 * i + 1], c, -mc));
-            const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[2 * i], c, -mc));
-            const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[2 * i + 1], c, -mc));
-            l_a += e0; l_b += e1; l_a += e2; l_b += e3;
-            pk[i] = N::pack2(e0, e1);
-            pk[8 + i] = N::pack2(e2, e3);
+            for (int i = 0; i < 8; ++i) {
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], c, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i + 1], c, -mc));
+                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], c, -mc));
+                const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], c, -mc));
+                l_a[b] += e0; l_b[b] += e1; l_a[b] += e2; l_b[b] += e3;
+                pk[b][i] = N::pack2(e0, e1);
+                pk[b][8 + i] = N::pack2(e2, e3);
+            }
         }
     };
 
@@ -416,74 +439,84 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     auto steady = [&](auto KST, auto VST, int tile) __attribute__((always_inline)) {
         constexpr uint32_t ks = decltype(KST)::value * TILEB;
         constexpr uint32_t vs = decltype(VST)::value * TILEB;
-        u32x4 fr[NM];                              // operand fragments, in matrix-instruction order
+        u32x4 fr[NF];                              // operand fragments, in the order they are consumed
         auto fetch = [&](int n) __attribute__((always_inline)) {
             if (n < NPV) fr[n] = read_v(vs, n);
             else fr[n] = read_k(ks, n - NPV);
         };
 #pragma unroll
         for (int n = 0; n < PD; ++n) fetch(n);
-        // the fragments are in flight; the row maximum needs no matrix instruction and covers their latency
-        if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, 32, tile) == 1) apply_mask(tile);
-        float mx = fmaxf(s0[0], s1[0]);
+        // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
+        if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile) == 1) apply_mask(tile);
+        bool moved[RB];
+        float alpha[RB], nmc[RB];
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, s0[r]), s1[r]);
-        mx = fmaxf(mx, swap_halves(mx));
-        bool moved;
-        const float alpha = new_reference(mx, moved);
-        const float mc = (m_run == -INFINITY) ? 0.0f : m_run * c;
-        uint32_t pn[16];                           // P(tile), becomes pk at the end
-        f32x16 n0, n1;                             // S^T(tile+1)
+        for (int b = 0; b < RB; ++b) {
+            alpha[b] = new_reference(b, row_max(b), moved[b]);
+            nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * c;
+        }
+        uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
+        f32x16 nx[RB][2];                          // S^T(tile+1)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int g = 0; g < NM; ++g) {
-            if (g + PD < NM) fetch(g + PD);
-            if (g < NPV) {
-                const int t2 = g / DB, db = g % DB;
-                const u32x4 pb = {pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
-                o[db] = N::mfma(fr[g], pb, o[db]);
-            } else {
-                const int n = g - NPV;
-                const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                if (n & 1) n1 = N::mfma(fr[g], qf[n >> 1], n < 2 ? zero : n1);
-                else n0 = N::mfma(fr[g], qf[n >> 1], n < 2 ? zero : n0);
-            }
-            // softmax work riding along: 16 element pairs spread over the NM matrix instructions
-            constexpr int PAIRS = 16;
-            const int e_begin = (g * PAIRS) / NM, e_end = ((g + 1) * PAIRS) / NM;
+        for (int g = 0; g < NF; ++g) {
+            if (g + PD < NF) fetch(g + PD);
 #pragma unroll
-            for (int e = e_begin; e < e_end; ++e) {
-                // pair e: elements (2e, 2e+1) of s0 for e < 8, of s1 for e >= 8.  The two empty asm
-                // statements pin the arithmetic between the surrounding matrix instructions: without them
-                // the compiler sinks all of it to the end of the iteration.
-                float x0 = e < 8 ? s0[2 * e] : s1[2 * (e - 8)];
-                float x1 = e < 8 ? s0[2 * e + 1] : s1[2 * (e - 8) + 1];
-                asm volatile("" : "+v"(x0), "+v"(x1));
-                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, -mc));
-                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, -mc));
-                l_a += e0;
-                l_b += e1;
-                uint32_t packed = N::pack2(e0, e1);
-                asm volatile("" : "+v"(packed), "+v"(l_a), "+v"(l_b));
-                pn[e] = packed;
+            for (int b = 0; b < RB; ++b) {
+                if (g < NPV) {
+                    const int t2 = g / DB, db = g % DB;
+                    o[b][db] = N::mfma(fr[g], p_operand(b, t2), o[b][db]);
+                } else {
+                    const int n = g - NPV;
+                    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n < 2 ? zero : nx[b][n & 1]);
+                }
+                // softmax work riding along: the 16*RB element pairs of this tile spread over the NF*RB matrix
+                // instructions, row block 0 first (its registers are free again when S^T(tile+1) is born)
+                constexpr int PAIRS = 16 * RB, SLOTS = NF * RB;
+                const int slot = g * RB + b;
+                const int p_begin = (slot * PAIRS) / SLOTS, p_end = ((slot + 1) * PAIRS) / SLOTS;
+#pragma unroll
+                for (int pi = p_begin; pi < p_end; ++pi) {
+                    // pair e of row block pb: elements (2e, 2e+1) of key block 0 for e < 8, of key block 1 for
+                    // e >= 8.  The two empty asm statements pin the arithmetic between the surrounding matrix
+                    // instructions (without them the compiler sinks all of it to the end of the iteration);
+                    // the first goes through the subtrahend, which stays in one register, so it costs no move.
+                    const int pb = pi / 16, e = pi % 16;
+                    const float x0 = e < 8 ? sx[pb][0][2 * e] : sx[pb][1][2 * (e - 8)];
+                    const float x1 = e < 8 ? sx[pb][0][2 * e + 1] : sx[pb][1][2 * (e - 8) + 1];
+                    asm volatile("" : "+v"(nmc[pb]));
+                    const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, nmc[pb]));
+                    const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, nmc[pb]));
+                    l_a[pb] += e0;
+                    l_b[pb] += e1;
+                    uint32_t packed = N::pack2(e0, e1);
+                    asm volatile("" : "+v"(packed), "+v"(l_a[pb]), "+v"(l_b[pb]));
+                    pn[pb][e] = packed;
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
-        if (moved) scale_o(alpha);                 // rare; PV(tile-1) has been issued in full by now
 #pragma unroll
-        for (int i = 0; i < 16; ++i) pk[i] = pn[i];
-        s0 = n0;
-        s1 = n1;
+        for (int b = 0; b < RB; ++b) {
+            if (moved[b]) scale_o(b, alpha[b]);    // rare; PV(tile-1) has been issued in full by now
+#pragma unroll
+            for (int i = 0; i < 16; ++i) pk[b][i] = pn[b][i];
+            sx[b][0] = nx[b][0];
+            sx[b][1] = nx[b][1];
+        }
     };
 
     // ---- prologue: K(t0) .. K(t0+LA-1) resident before the first iteration
     issue_k(t0, 0);
     if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
     wait_vm<0>();
-#pragma unroll
     // Q has landed too (vmcnt is 0).  Touching the fragments here lets the compiler see that, so that it places
     // no vmcnt wait of its own inside the loop, where it would also wait for the asynchronous tile loads.
-    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[b][s]));
     phase_barrier();
 
     // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST
@@ -538,22 +571,27 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead
     const bool faithful = MASKED && a.R == 0 && q0 == 0;
-    if (wave_live && !(faithful && wave == 0)) {
+    if (wave_live) {
         // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides)
-        const float l_half = l_a + l_b;
-        const float l_tot = l_half + swap_halves(l_half);
-        const float inv = 1.0f / l_tot;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+        for (int b = 0; b < RB; ++b) {
+            if (faithful && wave == 0 && b == 0) continue;
+            const int q = my_q + 32 * b;
+            const float l_half = l_a[b] + l_b[b];
+            const float l_tot = l_half + swap_halves(l_half);
+            const float inv = 1.0f / l_tot;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 w;
-                w[0] = N::pack2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv);
-                w[1] = N::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-                *reinterpret_cast<u32x2 *>(Oh + (size_t)my_q * D + 32 * db + 8 * g + 4 * half) = w;
-            }
-        if (a.lse != nullptr && half == 0)
-            a.lse[(size_t)bh * S + my_q] = m_run * a.scale + __builtin_logf(l_tot);
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
+                    w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2 *>(Oh + (size_t)q * D + 32 * db + 8 * g + 4 * half) = w;
+                }
+            if (a.lse != nullptr && half == 0)
+                a.lse[(size_t)bh * S + q] = m_run[b] * a.scale + __builtin_logf(l_tot);
+        }
     }
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
@@ -563,25 +601,29 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
 
 }  // namespace
 
-template <bool BF16, int D, bool MASKED, int NW, int NST>
+template <bool BF16, int D, bool MASKED, int NW, int RB, int NST>
 static hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
     const size_t smem = 2 * NST * TILEB;
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, NW, NST>;
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, NW, RB, NST>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
     return hipGetLastError();
 }
 
-// waves = 8: 256 query rows per workgroup, three LDS stages, one workgroup per CU.
-// waves = 4: 128 query rows per workgroup, two LDS stages, two workgroups per CU.
-hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int waves, unsigned grid, hipStream_t stream)
+// shape 0: 8 waves x 32 rows = 256 query rows per workgroup, three LDS stages, one workgroup per CU.
+// shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
+// (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
+// answers it with about 500 AGPR<->VGPR moves per tile.)
+hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
 #define FA_CASE(BF, DD, MK) \
-    if (bf16 == BF && D == DD && masked == MK) \
-        return waves == 8 ? launch<BF != 0, DD, MK != 0, 8, 3>(a, grid, stream) : launch<BF != 0, DD, MK != 0, 4, 2>(a, grid, stream);
+    if (bf16 == BF && D == DD && masked == MK) { \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, 8, 1, 3>(a, grid, stream); \
+        return launch<BF != 0, DD, MK != 0, 4, 1, 2>(a, grid, stream); \
+    }
     FA_CASE(0, 64, 0) FA_CASE(0, 64, 1) FA_CASE(0, 128, 0) FA_CASE(0, 128, 1)
     FA_CASE(1, 64, 0) FA_CASE(1, 64, 1) FA_CASE(1, 128, 0) FA_CASE(1, 128, 1)
 #undef FA_CASE
