@@ -42,7 +42,7 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline sample; 0 disables")
     ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
-    ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2), help="0 library default, 1 dispatch, 2 persistent")
+    ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2, 3), help="0 library default, 1 dispatch, 2 persistent snake, 3 persistent queue")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters to bytes)")

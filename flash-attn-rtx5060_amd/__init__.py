@@ -37,7 +37,7 @@ FA_ERR_NO_DEVICE = -9
 FA_ERR_TOO_LARGE = -10
 FA_DTYPE_F16 = 0
 FA_DTYPE_BF16 = 1
-FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT = 0, 1, 2
+FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT, FA_SCHED_QUEUE = 0, 1, 2, 3
 FA_TILE_SKIP, FA_TILE_PARTIAL, FA_TILE_FULL = 0, 1, 2
 
 #: every symbol include/fa_fwd.h declares

@@ -10,11 +10,16 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "fa_fwd.h"
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
 hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream);
+hipError_t fa_work_queue_base(unsigned **base);
+int fa_work_queue_slots();
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -30,6 +35,30 @@ int waves_for(int B, int N, int S)
 }
 
 thread_local char g_last_error[256] = "";
+
+// device address of the work-queue array, per device (every device holds its own copy of the symbol)
+constexpr int kMaxDevices = 64;
+std::mutex g_queue_mutex;
+unsigned *g_queue_base[kMaxDevices] = {};
+std::atomic<unsigned> g_queue_ticket{0};
+
+hipError_t work_queue_for_launch(unsigned **queue)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    {
+        std::lock_guard<std::mutex> lock(g_queue_mutex);
+        if (g_queue_base[dev] == nullptr) {
+            e = fa_work_queue_base(&g_queue_base[dev]);
+            if (e != hipSuccess) return e;
+        }
+    }
+    const unsigned slot = g_queue_ticket.fetch_add(1u) % (unsigned)fa_work_queue_slots();
+    *queue = g_queue_base[dev] + 16u * slot;
+    return hipSuccess;
+}
 
 int device_fail(hipError_t e, const char *what)
 {
@@ -161,7 +190,9 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     // free up, which is a longest-first greedy schedule.  Persistent mode launches one resident set of
     // workgroups that walk the list themselves.
     long long grid = a.n_items;
-    if (p->sched == FA_SCHED_PERSISTENT) {
+    a.queue = nullptr;
+    const int sched = p->sched == FA_SCHED_AUTO ? FA_SCHED_QUEUE : p->sched;
+    if (sched == FA_SCHED_PERSISTENT || sched == FA_SCHED_QUEUE) {
         int cus = kComputeUnits;
         int dev = 0;
         if (hipGetDevice(&dev) == hipSuccess) {
@@ -170,6 +201,10 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         }
         const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
         if (grid > resident) grid = resident;
+        if (sched == FA_SCHED_QUEUE) {
+            hipError_t qe = work_queue_for_launch(&a.queue);
+            if (qe != hipSuccess) return device_fail(qe, "work queue");
+        }
     }
     const int shape = waves == 8 ? 0 : 1;
     hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));

@@ -239,14 +239,43 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
 
-    // Work items.  A dispatch-mode grid has one workgroup per item (a single pass).  A persistent grid walks
-    // the longest-first list as a snake: pass 0 forwards, pass 1 backwards, ... so that every workgroup pairs
-    // long items with short ones; with a grid that is a multiple of 8 a workgroup also stays on the head
-    // lane of its XCD.
+    // Work items.  Without a queue the grid is static: one workgroup per item (a single pass), or a resident
+    // grid that walks the longest-first list as a snake (pass 0 forwards, pass 1 backwards, ...), pairing
+    // long items with short ones.  With a queue, a resident grid takes items dynamically: a workgroup on XCD x
+    // takes list positions x, x+8, x+16, ... from that XCD's counter, so a head stays on one XCD's L2 and a
+    // workgroup that finishes early simply takes the next item -- the hardware dispatcher's longest-first
+    // greedy schedule without its workgroup launch gaps (about 10 us per item on this chip).
     const int G = (int)gridDim.x;
-    for (int pass = 0; (long long)pass * G < a.n_items; ++pass) {
-    const long long item = (long long)pass * G + ((pass & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x);
-    if (item >= a.n_items) continue;
+    unsigned xcd = 0;
+    if (a.queue != nullptr) {
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcd));
+        xcd &= 7u;
+    }
+    volatile unsigned *next_slot = reinterpret_cast<volatile unsigned *>(smem + 2 * NST * TILEB);
+    for (int pass = 0;; ++pass) {
+    long long item;
+    if (a.queue == nullptr) {
+        if ((long long)pass * G >= a.n_items) break;
+        item = (long long)pass * G + ((pass & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x);
+        if (item >= a.n_items) continue;
+    } else {
+        if (tid == 0) {
+            // own XCD's list first; when that is exhausted, help the others (this also makes the result
+            // independent of how the hardware spreads the workgroups over the XCDs)
+            unsigned found = 0xffffffffu;
+            for (unsigned xo = 0; xo < 8u && found == 0xffffffffu; ++xo) {
+                const unsigned xq = (xcd + xo) & 7u;
+                const long long cand = (long long)atomicAdd(&a.queue[xq], 1u) * 8 + xq;
+                if (cand < a.n_items) found = (unsigned)cand;
+            }
+            *next_slot = found;
+        }
+        __syncthreads();
+        const unsigned taken = *next_slot;
+        __syncthreads();
+        if (taken == 0xffffffffu) break;
+        item = (long long)taken;
+    }
     int bh, qblock;
     fa_item_decode(item, a.BH, a.n_qblocks, a.descending, &bh, &qblock);
     const int S = a.S;
@@ -597,15 +626,35 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
                                      reinterpret_cast<float *>(smem));
     }   // next work item
+    // the last workgroup to leave rewinds the queue for the next launch that uses it
+    if (a.queue != nullptr && tid == 0) {
+        __threadfence();
+        if (atomicAdd(&a.queue[8], 1u) == (unsigned)G - 1u) {
+#pragma unroll
+            for (int x = 0; x < 9; ++x) a.queue[x] = 0u;
+        }
+    }
 }
 
 }  // namespace
+
+// Work queues of FA_SCHED_QUEUE launches: kQueueSlots sets of nine counters, all zero between launches (the
+// last workgroup of a launch rewinds its set).  Launches take the sets round-robin, so launches that overlap
+// on one device do not share a set unless more than kQueueSlots of them are in flight at once.
+constexpr int kQueueSlots = 32;
+static __device__ __align__(256) unsigned g_work_queues[kQueueSlots][16];
+
+hipError_t fa_work_queue_base(unsigned **base)
+{
+    return hipGetSymbolAddress(reinterpret_cast<void **>(base), HIP_SYMBOL(g_work_queues));
+}
+int fa_work_queue_slots() { return kQueueSlots; }
 
 template <bool BF16, int D, bool MASKED, int NW, int RB, int NST>
 static hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
-    const size_t smem = 2 * NST * TILEB;
+    const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
     auto kern = fa_fwd_pipelined<BF16, D, MASKED, NW, RB, NST>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;

@@ -21,6 +21,7 @@ struct FaKernelArgs {
     float scale;         // softmax scale
     float scale_log2e;   // softmax scale * log2(e)
     long long n_items;   // work items: BH * n_qblocks
+    unsigned *queue;     // null, or 9 counters of a work queue: next list position per XCD [0..7], finished workgroups [8]
 };
 
 #endif

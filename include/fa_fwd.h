@@ -40,9 +40,12 @@ enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
 
 /* How work items (batch, head, query block) reach the compute units. */
 enum {
-    FA_SCHED_AUTO = 0,        /* the library picks (currently FA_SCHED_DISPATCH)              */
+    FA_SCHED_AUTO = 0,        /* the library picks (currently FA_SCHED_QUEUE)                 */
     FA_SCHED_DISPATCH = 1,    /* one workgroup per work item, launched longest-first          */
-    FA_SCHED_PERSISTENT = 2   /* a resident grid sized to the CUs walks the longest-first list */
+    FA_SCHED_PERSISTENT = 2,  /* a resident grid sized to the CUs walks the longest-first list
+                                 in a fixed snake order                                       */
+    FA_SCHED_QUEUE = 3        /* a resident grid takes items from the longest-first list
+                                 through per-XCD counters in the library's own device memory  */
 };
 
 /*
