@@ -271,7 +271,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             *next_slot = found;
         }
         __syncthreads();
-        const unsigned taken = *next_slot;
+        // uniform by construction: say so, or everything derived from the item lives in vector registers
+        const unsigned taken = (unsigned)__builtin_amdgcn_readfirstlane((int)*next_slot);
         __syncthreads();
         if (taken == 0xffffffffu) break;
         item = (long long)taken;
