@@ -140,8 +140,9 @@ def host_lib():
 
 
 def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
-                window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO):
+                window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0):
     p = FaFwdParams()
+    p.alibi_slopes_ptr = alibi_ptr or None
     p.Q, p.K, p.V, p.O, p.L = q_ptr or None, k_ptr or None, v_ptr or None, o_ptr or None, lse_ptr or None
     p.B, p.N, p.S, p.d = B, N, S, d
     p.softmax_scale = (1.0 / math.sqrt(d)) if softmax_scale is None else softmax_scale
@@ -151,8 +152,9 @@ def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softm
 
 
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                            return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO):
-    """O, LSE = attention(q, k, v) on the GPU through fa_fwd(); torch tensors [B, N, S, d]."""
+                            return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None):
+    """O, LSE = attention(q, k, v) on the GPU through fa_fwd(); torch tensors [B, N, S, d].
+    ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26)."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise ValueError("q, k, v must live on the GPU")
@@ -163,13 +165,17 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
     if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
         raise ValueError("q, k, v must be contiguous [B, N, S, d]")
     B, N, S, d = q.shape
+    if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
+                                         and alibi_slopes.is_contiguous() and tuple(alibi_slopes.shape) == (N,)):
+        raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
     if out is None:
         out = torch.empty_like(q)
     if return_lse and lse is None:
         lse = torch.empty((B, N, S), dtype=torch.float32, device=q.device)
     p = make_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                     lse.data_ptr() if return_lse else 0, softmax_scale, causal, window_left, window_right,
-                    FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched)
+                    FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched,
+                    0 if alibi_slopes is None else alibi_slopes.data_ptr())
     stream = torch.cuda.current_stream(q.device).cuda_stream
     st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
     if st != FA_OK:

@@ -77,7 +77,7 @@ const char *fa_strerror(int status)
     case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
     case FA_ERR_SEQLEN_MULTIPLE: return "seqlen must be a multiple of 128";
-    case FA_ERR_UNSUPPORTED: return "dropout and ALiBi are not supported";
+    case FA_ERR_UNSUPPORTED: return "dropout is not supported";
     case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
     case FA_ERR_SCALE: return "softmax_scale must be finite and positive";
     case FA_ERR_DEVICE: return "HIP runtime error";
@@ -156,7 +156,7 @@ int fa_fwd_validate(const fa_fwd_params *p)
     if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
     if (p->S % 128 != 0) return FA_ERR_SEQLEN_MULTIPLE;
     if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
-    if (p->dropout_prob != 0.0f || p->states != nullptr || p->alibi_slopes_ptr != nullptr) return FA_ERR_UNSUPPORTED;
+    if (p->dropout_prob != 0.0f || p->states != nullptr) return FA_ERR_UNSUPPORTED;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
@@ -174,6 +174,8 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.V = static_cast<const uint16_t *>(p->V);
     a.O = static_cast<uint16_t *>(p->O);
     a.lse = p->L;
+    a.alibi = p->alibi_slopes_ptr;
+    a.H = p->N;
     a.BH = p->B * p->N;
     a.S = p->S;
     const int waves = waves_for(p->B, p->N, p->S);
@@ -218,8 +220,8 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
 {
     (void)M;
     (void)states;
-    (void)alibi_slopes;
-    if (Is_dropout || Has_alibi) return FA_ERR_UNSUPPORTED;
+    if (Is_dropout) return FA_ERR_UNSUPPORTED;
+    if (Has_alibi && alibi_slopes == nullptr) return FA_ERR_NULL_POINTER;
     if (d <= 0) return FA_ERR_HEAD_DIM;
     fa_fwd_params p;
     memset(&p, 0, sizeof(p));
@@ -228,6 +230,7 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
     p.B = B; p.N = N; p.S = S; p.d = d;
     p.softmax_scale = (float)(1.0 / sqrt((double)d));      // flash_forward.h:639
     p.dropout_prob = dropout_prob;
+    p.alibi_slopes_ptr = Has_alibi ? alibi_slopes : nullptr;      // [N] device floats, main.cu:36-45
     p.window_size_left = Is_local ? window_size : -1;      // flash_forward.h:640-641, mask.h:55
     p.window_size_right = Is_local ? window_size : -1;
     if (Is_local && window_size < 0) { p.window_size_left = p.window_size_right = 0; }

@@ -160,7 +160,8 @@ template <bool BF16> __device__ __forceinline__ float storage_product(float a, f
 
 template <bool BF16, int D>
 __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
-                                    float *lse_h, int S, int L, float scale, float *sc /* LDS, 32*32 floats */)
+                                    float *lse_h, int S, int L, float scale, float slope,
+                                    float *sc /* LDS, 32*32 floats */)
 {
     constexpr int R = kFaithfulRows;
     const int rows = S < R ? S : R;
@@ -174,6 +175,8 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
             for (int t = 0; t < D; ++t)
                 sum += storage_product<BF16>(storage_to_f32<BF16>(Qh[(size_t)i * D + t]), storage_to_f32<BF16>(Kh[(size_t)j * D + t]));
             s = sum * scale;
+            // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
+            if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(i - j)));
         }
         sc[idx] = s;
     }
@@ -210,7 +213,7 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, int NW, int RB, int NST>
 __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
 {
     constexpr int WR = 32 * RB;                   // query rows per wave
@@ -349,8 +352,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
 #pragma unroll
     for (int b = 0; b < RB; ++b) { m_run[b] = -INFINITY; l_a[b] = 0.0f; l_b[b] = 0.0f; }
+    // Without ALiBi the tile scores stay raw dot products and the softmax scale is folded into the exponent
+    // (exp2(s*c - m*c)).  With ALiBi a tile is first rewritten in place to log2 units with the bias applied,
+    // s*c - slope*log2(e)*|i-j| (mask.h:21-26 subtracts slope*|i-j| from the scaled score), so maxima, the
+    // reference point and the exponent work on those values with a factor of one.
     const float c = a.scale_log2e;
-    const float thresh = kRescaleLog2 / c;
+    const float cs = ALIBI ? 1.0f : c;
+    const float slope = ALIBI ? a.alibi[bh % a.H] : 0.0f;
+    const float slope_l2 = slope * 1.44269504088896340736f;
+    const float thresh = kRescaleLog2 / cs;
     uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
     f32x16 sx[RB][2];           // S^T of the tile whose softmax comes next: [key block 0 / 1]
 
@@ -377,6 +387,19 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             }
         }
     };
+    auto apply_alibi = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            // signed distance of this lane's query to the lane's first key of the tile: exact in fp32
+            const float base = (float)(my_q + 32 * b - (tile * kBlockKeys + 4 * half));
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float k0 = (float)(8 * (r >> 2) + (r & 3));
+                sx[b][0][r] = __builtin_fmaf(__builtin_fabsf(base - k0), -slope_l2, sx[b][0][r] * c);
+                sx[b][1][r] = __builtin_fmaf(__builtin_fabsf(base - (k0 + 32.0f)), -slope_l2, sx[b][1][r] * c);
+            }
+        }
+    };
     auto row_max = [&](int b) __attribute__((always_inline)) {
         float mx = fmaxf(sx[b][0][0], sx[b][1][0]);
 #pragma unroll
@@ -391,7 +414,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         moved = __builtin_amdgcn_ballot_w64(grow) != 0;
         if (moved) {
             const float m_new = grow ? mx : m_run[b];
-            alpha = (m_run[b] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run[b] - m_new) * c);
+            alpha = (m_run[b] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run[b] - m_new) * cs);
             l_a[b] *= alpha;
             l_b[b] *= alpha;
             m_run[b] = m_new;
@@ -445,19 +468,20 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
     };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
+        if (ALIBI) apply_alibi(tile);
         if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile) == 1) apply_mask(tile);
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             bool moved;
             const float alpha = new_reference(b, row_max(b), moved);
             if (moved) scale_o(b, alpha);
-            const float mc = (m_run[b] == -INFINITY) ? 0.0f : m_run[b] * c;
+            const float mc = (m_run[b] == -INFINITY) ? 0.0f : m_run[b] * cs;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], c, -mc));
-                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i + 1], c, -mc));
-                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], c, -mc));
-                const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], c, -mc));
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], cs, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i + 1], cs, -mc));
+                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], cs, -mc));
+                const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], cs, -mc));
                 l_a[b] += e0; l_b[b] += e1; l_a[b] += e2; l_b[b] += e3;
                 pk[b][i] = N::pack2(e0, e1);
                 pk[b][8 + i] = N::pack2(e2, e3);
@@ -477,13 +501,14 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int n = 0; n < PD; ++n) fetch(n);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
+        if (ALIBI) apply_alibi(tile);
         if (MASKED && fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile) == 1) apply_mask(tile);
         bool moved[RB];
         float alpha[RB], nmc[RB];
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             alpha[b] = new_reference(b, row_max(b), moved[b]);
-            nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * c;
+            nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * cs;
         }
         uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
         f32x16 nx[RB][2];                          // S^T(tile+1)
@@ -516,8 +541,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     const float x0 = e < 8 ? sx[pb][0][2 * e] : sx[pb][1][2 * (e - 8)];
                     const float x1 = e < 8 ? sx[pb][0][2 * e + 1] : sx[pb][1][2 * (e - 8) + 1];
                     asm volatile("" : "+v"(nmc[pb]));
-                    const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, nmc[pb]));
-                    const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, nmc[pb]));
+                    const float e0 = __builtin_amdgcn_exp2f(ALIBI ? x0 + nmc[pb] : __builtin_fmaf(x0, c, nmc[pb]));
+                    const float e1 = __builtin_amdgcn_exp2f(ALIBI ? x1 + nmc[pb] : __builtin_fmaf(x1, c, nmc[pb]));
                     l_a[pb] += e0;
                     l_b[pb] += e1;
                     uint32_t packed = N::pack2(e0, e1);
@@ -620,12 +645,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     *reinterpret_cast<u32x2 *>(Oh + (size_t)q * D + 32 * db + 8 * g + 4 * half) = w;
                 }
             if (a.lse != nullptr && half == 0)
-                a.lse[(size_t)bh * S + q] = m_run[b] * a.scale + __builtin_logf(l_tot);
+                a.lse[(size_t)bh * S + q] = m_run[b] * (ALIBI ? 0.69314718055994530942f : a.scale) + __builtin_logf(l_tot);
         }
     }
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
-                                     reinterpret_cast<float *>(smem));
+                                     slope, reinterpret_cast<float *>(smem));
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
     if (a.queue != nullptr && tid == 0) {
@@ -651,12 +676,12 @@ hipError_t fa_work_queue_base(unsigned **base)
 }
 int fa_work_queue_slots() { return kQueueSlots; }
 
-template <bool BF16, int D, bool MASKED, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, int NW, int RB, int NST>
 static hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
     const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, NW, RB, NST>;
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, NW, RB, NST>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
@@ -669,13 +694,15 @@ static hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t strea
 // answers it with about 500 AGPR<->VGPR moves per tile.)
 hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
-#define FA_CASE(BF, DD, MK) \
-    if (bf16 == BF && D == DD && masked == MK) { \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, 8, 1, 3>(a, grid, stream); \
-        return launch<BF != 0, DD, MK != 0, 4, 1, 2>(a, grid, stream); \
+    const int alibi = a.alibi != nullptr;
+#define FA_CASE(BF, DD, MK, AL) \
+    if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, 8, 1, 3>(a, grid, stream); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, 4, 1, 2>(a, grid, stream); \
     }
-    FA_CASE(0, 64, 0) FA_CASE(0, 64, 1) FA_CASE(0, 128, 0) FA_CASE(0, 128, 1)
-    FA_CASE(1, 64, 0) FA_CASE(1, 64, 1) FA_CASE(1, 128, 0) FA_CASE(1, 128, 1)
+#define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
+    FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)
+#undef FA_CASES
 #undef FA_CASE
     return hipErrorInvalidValue;
 }

@@ -12,6 +12,8 @@ struct FaKernelArgs {
     const uint16_t *V;
     uint16_t *O;
     float *lse;          // may be null
+    const float *alibi;  // per-head ALiBi slopes [H], or null
+    int H;               // heads per batch entry
     int BH;              // batch * heads
     int S;
     int n_qblocks;       // query blocks per head

@@ -30,7 +30,7 @@
 #define PEAK_TFLOPS 2516.6 /* 256 CU x 4096 FLOP/clk x 2.4 GHz, dense fp16 = bf16 */
 
 typedef struct {
-    int B, N, S, d, bf16, causal, wl, wr, iters, warmup, threads, lse;
+    int B, N, S, d, bf16, causal, wl, wr, iters, warmup, threads, lse, alibi;
     unsigned long long seed;
     float sigma, scale;
     double row_fraction;
@@ -107,6 +107,7 @@ int main(int argc, char **argv)
         else if (!strcmp(a, "--threads")) { NEED_VALUE(); c.threads = atoi(v); }
         else if (!strcmp(a, "--dump")) { NEED_VALUE(); c.dump = v; }
         else if (!strcmp(a, "--no-lse")) c.lse = 0;
+        else if (!strcmp(a, "--alibi")) c.alibi = 1;
         else { fprintf(stderr, "unknown argument %s\n", a); return 2; }
     }
     if (!scale_given && c.d > 0) c.scale = (float)(1.0 / sqrt((double)c.d));
@@ -145,6 +146,16 @@ int main(int argc, char **argv)
     p.window_size_left = c.wl; p.window_size_right = c.wr;
     p.dtype = c.bf16 ? FA_DTYPE_BF16 : FA_DTYPE_F16;
     p.is_causal = c.causal;
+    float *hs = NULL;
+    void *ds = NULL;
+    if (c.alibi) {      /* the slopes of main.cu:36-45: -2^(-8/N * (h+1)), copied to the device */
+        hs = malloc((size_t)c.N * sizeof(float));
+        if (!hs) { fprintf(stderr, "host allocation failed\n"); return 1; }
+        for (int h = 0; h < c.N; ++h) hs[h] = (float)-pow(2.0, -8.0 / c.N * (h + 1));
+        if (check(fa_dev_malloc(&ds, (size_t)c.N * sizeof(float)), "alloc slopes") ||
+            check(fa_dev_h2d(ds, hs, (size_t)c.N * sizeof(float)), "H2D slopes")) return 1;
+        p.alibi_slopes_ptr = ds;
+    }
 
     for (int i = 0; i < c.warmup; ++i)
         if (check(fa_fwd(&p, NULL), "warm-up launch")) return 1;
@@ -170,11 +181,11 @@ int main(int argc, char **argv)
         if (!isfinite(x)) ++bad;                      /* main.cu:149 rejects NaN/Inf the same way */
     }
     printf("{\"config\": \"%s\", \"device\": \"%s\", \"compute_units\": %d, \"B\": %d, \"N\": %d, \"S\": %d, \"d\": %d, "
-           "\"dtype\": \"%s\", \"causal\": %d, \"window_left\": %d, \"window_right\": %d, \"scale\": %.9g, \"seed\": %llu, "
+           "\"dtype\": \"%s\", \"causal\": %d, \"window_left\": %d, \"window_right\": %d, \"alibi\": %d, \"scale\": %.9g, \"seed\": %llu, "
            "\"iters\": %d, \"ms_median\": %.6f, \"ms_min\": %.6f, \"algorithmic_flops\": %.6e, "
            "\"tflops_median\": %.3f, \"tflops_best\": %.3f, \"peak_tflops\": %.1f, \"frac_of_peak_median\": %.4f, "
            "\"nonfinite_outputs\": %zu}\n",
-           c.name, devname, cus, c.B, c.N, c.S, c.d, c.bf16 ? "bf16" : "fp16", c.causal, c.wl, c.wr, (double)c.scale,
+           c.name, devname, cus, c.B, c.N, c.S, c.d, c.bf16 ? "bf16" : "fp16", c.causal, c.wl, c.wr, c.alibi, (double)c.scale,
            c.seed, c.iters, med, best, flops, flops / med / 1e9, flops / best / 1e9, PEAK_TFLOPS,
            flops / med / 1e9 / PEAK_TFLOPS, bad);
 
@@ -183,9 +194,12 @@ int main(int argc, char **argv)
         rc |= dump_file(c.dump, "q.bin", hq, bytes) | dump_file(c.dump, "k.bin", hk, bytes) |
               dump_file(c.dump, "v.bin", hv, bytes) | dump_file(c.dump, "o.bin", ho, bytes);
         if (c.lse) rc |= dump_file(c.dump, "lse.bin", hl, rows * sizeof(float));
+        if (c.alibi) rc |= dump_file(c.dump, "slopes.bin", hs, (size_t)c.N * sizeof(float));
     }
     fa_event_destroy(e0); fa_event_destroy(e1);
     fa_dev_free(dq); fa_dev_free(dk); fa_dev_free(dv); fa_dev_free(dO); fa_dev_free(dl);
+    if (ds) fa_dev_free(ds);
+    free(hs);
     free(hq); free(hk); free(hv); free(ho); free(hl); free(ms);
     return rc;
 }

@@ -28,7 +28,7 @@ enum {
     FA_ERR_BAD_SHAPE = -2,         /* B, N or S is not positive                              */
     FA_ERR_HEAD_DIM = -3,          /* d not in {64, 128}: reference throws, flash_forward.h:587 */
     FA_ERR_SEQLEN_MULTIPLE = -4,   /* S % 128 != 0: reference assumes it silently, :134,637  */
-    FA_ERR_UNSUPPORTED = -5,       /* dropout or ALiBi requested                             */
+    FA_ERR_UNSUPPORTED = -5,       /* dropout requested                                      */
     FA_ERR_DTYPE = -6,             /* dtype is neither FA_DTYPE_F16 nor FA_DTYPE_BF16        */
     FA_ERR_SCALE = -7,             /* softmax_scale is not a finite positive number          */
     FA_ERR_DEVICE = -8,            /* a HIP runtime call failed; see fa_last_device_error()  */
@@ -74,7 +74,7 @@ typedef struct fa_fwd_params {
     void *states;             /* dropout RNG states: must be NULL                             */
     int window_size_left;     /* keys with i - j > left are masked;  < 0 = unbounded          */
     int window_size_right;    /* keys with j - i > right are masked; < 0 = unbounded          */
-    const float *alibi_slopes_ptr; /* must be NULL                                            */
+    const float *alibi_slopes_ptr; /* [N] device floats: score -= slope[h]*|i-j| (mask.h:21-26), or NULL */
     int split_num;            /* unused, as in the reference (utils.h:164)                    */
     /* --- beyond mykernelParamType --- */
     int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                 */
@@ -100,7 +100,9 @@ int fa_fwd(const fa_fwd_params *p, void *stream);
  * Like the reference it runs on the default stream of the current device and
  * returns after the kernel has finished (flash_forward.h:655); unlike it, it
  * prints nothing, returns a status, and fills L with the fp32 logsumexp when
- * L is non-NULL.  M is ignored.  Dropout and ALiBi return FA_ERR_UNSUPPORTED.
+ * L is non-NULL.  M is ignored.  `Has_alibi` takes `alibi_slopes` as N device floats and subtracts
+ * slope[h]*|i-j| from every scaled score, once (mask.h:21-26; the reference applies it twice when causal
+ * and local are both set).  Dropout returns FA_ERR_UNSUPPORTED.
  */
 int run_flash_attention(int B, int N, int S, int d,
                         void *Q, void *K, void *V, void *O,

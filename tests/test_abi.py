@@ -70,7 +70,7 @@ def test_validate_status_codes(fa):
     assert status(softmax_scale=float("inf")) == fa.FA_ERR_SCALE
     assert status_raw(dict(dropout_prob=0.1)) == fa.FA_ERR_UNSUPPORTED
     assert status_raw(dict(states=0x10)) == fa.FA_ERR_UNSUPPORTED
-    assert status_raw(dict(alibi_slopes_ptr=0x10)) == fa.FA_ERR_UNSUPPORTED
+    assert status_raw(dict(alibi_slopes_ptr=0x10)) == fa.FA_OK               # ALiBi slopes are accepted
     assert status(B=70000, N=70000, S=128) == fa.FA_ERR_TOO_LARGE
     # fa_fwd itself refuses the same blocks before touching any device
     p = fa.make_params(**dict(ok, d=96))
@@ -81,7 +81,7 @@ def test_reference_entry_point_rejects_unsupported_flags(fa):
     L = fa.lib()
     args = [2, 8, 2048, 64, 0x1000, 0x2000, 0x3000, 0x4000, None, None]
     assert L.run_flash_attention(*args, 1, 0, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_UNSUPPORTED   # dropout
-    assert L.run_flash_attention(*args, 0, 0, 0, 1, 0, None, 0.0, None) == fa.FA_ERR_UNSUPPORTED   # ALiBi
+    assert L.run_flash_attention(*args, 0, 0, 0, 1, 0, None, 0.0, None) == fa.FA_ERR_NULL_POINTER  # ALiBi without slopes
     bad = list(args)
     bad[3] = 48
     assert L.run_flash_attention(*bad, 0, 0, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_HEAD_DIM

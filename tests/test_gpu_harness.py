@@ -16,6 +16,8 @@ pytestmark = pytest.mark.gpu
     (["--config", "c1"], (1, 4, 256, 64), 0, False, -1, 27),
     (["--B", "2", "--N", "3", "--S", "1024", "--d", "128", "--bf16", "--causal", "--window-left", "200", "--seed", "5"],
      (2, 3, 1024, 128), 1, True, 200, 5),
+    (["--B", "1", "--N", "8", "--S", "1024", "--d", "64", "--causal", "--alibi", "--seed", "6"],
+     (1, 8, 1024, 64), 0, True, -1, 6),
 ])
 def test_harness_output_matches_oracle(fa, oracle, tmp_path, args, shape, dtype, causal, wl, seed):
     assert os.path.exists(fa.HARNESS_PATH), "fa_harness has not been built"
@@ -34,6 +36,10 @@ def test_harness_output_matches_oracle(fa, oracle, tmp_path, args, shape, dtype,
     o = np.fromfile(f"{prefix}.o.bin", dtype=np.uint16).reshape(-1, D)
     lse = np.fromfile(f"{prefix}.lse.bin", dtype=np.float32)
     rows = sample_rows(shape, 1024, seed)
-    o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, causal, wl, -1)
+    slopes = None
+    if "--alibi" in args:       # the slopes of the reference's main() (src/main.cu:38-42)
+        slopes = np.fromfile(f"{prefix}.slopes.bin", dtype=np.float32)
+        assert np.array_equal(slopes, (-np.power(2.0, -8.0 / H * (np.arange(H) + 1))).astype(np.float32))
+    o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, causal, wl, -1, slopes)
     err = errors(oracle.to_f32(o[rows], dtype), oracle.to_f32(o_ref, dtype), lse[rows], lse_ref)
     assert_within(err, dtype, f"harness {args}")

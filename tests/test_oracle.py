@@ -283,6 +283,74 @@ def test_against_numpy_f64_and_torch_sdpa(dtype, causal, wl, wr):
     assert np.max(np.abs(lse - lse_np)) <= (2e-3 if dtype == F16 else 8e-3)   # bf16 products carry 2^-9 relative error
 
 
+# ---------------------------------------------------------------- ALiBi (main.cu:200-207)
+@pytest.mark.parametrize("causal", [False, True])
+def test_alibi_closed_form_zero_queries(causal):
+    """Q = 0 leaves only the bias: p_ij = exp(-slope_h |i-j|) / Z_i over the visible keys, and V = identity
+    makes O = P.  A bias with the wrong sign, a missing |.|, the wrong head's slope or a bias applied after the
+    mask's -inf would all change these numbers."""
+    H, S = 3, 48
+    slopes = np.array([0.5, -0.0625, 0.0], dtype=np.float32)      # both signs and a zero
+    q = np.zeros((1, H, S, S), dtype=np.uint16)
+    k = rand_bits(np.random.default_rng(3), (1, H, S, S), F16)
+    v = np.broadcast_to(ob.from_f32(np.eye(S, dtype=np.float32), F16), (1, H, S, S)).copy()
+    o, lse = ob.full(q, k, v, F16, None, causal, -1, -1, slopes)
+    o64, lse64 = ob.rows_f64(q, k, v, np.arange(H * S), F16, None, causal, -1, -1, slopes)
+    i, j = np.meshgrid(np.arange(S), np.arange(S), indexing="ij")
+    for h in range(H):
+        w = np.exp(-np.float64(slopes[h]) * np.abs(i - j))
+        if causal:
+            w = np.where(j <= i, w, 0.0)
+        # normalise against the row maximum like a softmax does (exp(+big) overflows nothing here, S is small)
+        Z = w.sum(axis=1, keepdims=True)
+        assert np.allclose(o64.reshape(H, S, S)[h], w / Z, atol=1e-12)
+        assert np.allclose(lse64.reshape(H, S)[h], np.log(Z[:, 0]), atol=1e-12)
+        assert np.max(np.abs(ob.to_f32(o, F16)[0, h] - w / Z)) <= 6e-4       # p rounded to fp16: half an ulp below 1
+        assert np.max(np.abs(lse[0, h] - np.log(Z[:, 0]))) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("causal,wl,wr", [(False, -1, -1), (True, -1, -1), (True, 24, -1), (False, 16, 16)])
+def test_alibi_against_numpy_f64_and_torch_sdpa(dtype, causal, wl, wr):
+    import torch
+    rng = np.random.default_rng(17)
+    shape = (2, 4, 128, 64)
+    B, H, S, D = shape
+    q, k, v = (rand_bits(rng, shape, dtype) for _ in range(3))
+    slopes = np.array([2.0 ** -1, 2.0 ** -3, -(2.0 ** -4), 2.0 ** -8], dtype=np.float32)
+    idx = np.arange(B * H * S)
+    o64, lse64 = ob.rows_f64(q, k, v, idx, dtype, None, causal, wl, wr, slopes)
+    i, j = np.meshgrid(np.arange(S), np.arange(S), indexing="ij")
+    vis = np.ones((S, S), dtype=bool)
+    if causal:
+        vis &= j <= i
+    if wl >= 0:
+        vis &= i - j <= wl
+    if wr >= 0:
+        vis &= j - i <= wr
+    bias = -slopes.astype(np.float64)[None, :, None, None] * np.abs(i - j)[None, None]
+    bias = np.where(vis[None, None], bias, -np.inf)
+    # numpy fp64, written out
+    qf, kf, vf = (ob.to_f32(x, dtype).astype(np.float64) for x in (q, k, v))
+    s = np.einsum("bhid,bhjd->bhij", qf, kf) * np.float64(np.float32(1 / np.sqrt(D))) + bias
+    mx = s.max(axis=-1, keepdims=True)
+    e = np.exp(s - mx)
+    l = e.sum(axis=-1, keepdims=True)
+    o_np, lse_np = np.einsum("bhij,bhjd->bhid", e / l, vf), (mx + np.log(l))[..., 0]
+    assert np.allclose(o64.reshape(shape), o_np, atol=1e-12)
+    assert np.allclose(lse64.reshape(shape[:3]), lse_np, atol=1e-12)
+    # a third-party library with the bias as an additive float mask
+    o_t = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(qf), torch.from_numpy(kf), torch.from_numpy(vf),
+        attn_mask=torch.from_numpy(np.broadcast_to(bias, (B, H, S, S)).copy()), scale=float(np.float32(1 / np.sqrt(D))))
+    assert np.allclose(o64.reshape(shape), o_t.numpy(), atol=1e-10)
+    # the reference-order fp32 path stays close to the exact result (a steep slope concentrates the softmax on a
+    # few keys, where the verifier's rounding of every p*v product to the storage type shows: up to 3e-3 in fp16)
+    o, lse = ob.full(q, k, v, dtype, None, causal, wl, wr, slopes)
+    assert np.max(np.abs(ob.to_f32(o, dtype) - o_np)) <= (3e-3 if dtype == F16 else 1.6e-2)
+    assert np.max(np.abs(lse - lse_np)) <= (2e-3 if dtype == F16 else 8e-3)
+
+
 def test_golden_fixture_f64():
     """tests/golden/attn_small_f64.npz was written by tests/golden/make_golden.py with a numpy fp64 brute force
     (no oracle code involved)."""
