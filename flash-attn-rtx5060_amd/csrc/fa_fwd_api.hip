@@ -31,7 +31,7 @@ constexpr int kComputeUnits = 256;      // MI355X; the persistent grid is sized 
 int waves_for(int B, int N, int S)
 {
     const long long big_items = (long long)B * N * ((S + 255) / 256);
-    return big_items >= 4LL * kComputeUnits ? 8 : 4;
+    return big_items >= 2LL * kComputeUnits ? 8 : 4;
 }
 
 thread_local char g_last_error[256] = "";
