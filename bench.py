@@ -21,8 +21,8 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 
 # HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
-# worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 551.7 MB read + 136.3 MB written.
-MEASURED_HBM_BYTES = {"c3": 688.0e6}
+# worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 424.1 MB read + 137.0 MB written.
+MEASURED_HBM_BYTES = {"c3": 561.1e6}
 
 WORKLOADS = {
     # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
