@@ -35,6 +35,7 @@ FA_ERR_SCALE = -7
 FA_ERR_DEVICE = -8
 FA_ERR_NO_DEVICE = -9
 FA_ERR_TOO_LARGE = -10
+FA_ERR_LAYOUT = -11
 FA_DTYPE_F16 = 0
 FA_DTYPE_BF16 = 1
 FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT, FA_SCHED_QUEUE = 0, 1, 2, 3
@@ -63,6 +64,9 @@ class FaFwdParams(ctypes.Structure):
         ("window_size_left", ctypes.c_int), ("window_size_right", ctypes.c_int),
         ("alibi_slopes_ptr", ctypes.c_void_p), ("split_num", ctypes.c_int),
         ("dtype", ctypes.c_int), ("is_causal", ctypes.c_int), ("sched", ctypes.c_int),
+        ("n_kv_heads", ctypes.c_int),
+        ("q_strides", ctypes.c_longlong * 3), ("k_strides", ctypes.c_longlong * 3),
+        ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
     ]
 
 
@@ -140,9 +144,15 @@ def host_lib():
 
 
 def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
-                window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0):
+                window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0,
+                n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None):
+    """A filled fa_fwd_params.  Strides are (batch, head, row) in elements, None = contiguous [B,N,S,d]."""
     p = FaFwdParams()
     p.alibi_slopes_ptr = alibi_ptr or None
+    p.n_kv_heads = n_kv_heads
+    for name, st in (("q_strides", q_strides), ("k_strides", k_strides), ("v_strides", v_strides), ("o_strides", o_strides)):
+        if st is not None:
+            setattr(p, name, (ctypes.c_longlong * 3)(*st))
     p.Q, p.K, p.V, p.O, p.L = q_ptr or None, k_ptr or None, v_ptr or None, o_ptr or None, lse_ptr or None
     p.B, p.N, p.S, p.d = B, N, S, d
     p.softmax_scale = (1.0 / math.sqrt(d)) if softmax_scale is None else softmax_scale
@@ -153,29 +163,36 @@ def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softm
 
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
                             return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None):
-    """O, LSE = attention(q, k, v) on the GPU through fa_fwd(); torch tensors [B, N, S, d].
+    """O, LSE = attention(q, k, v) on the GPU through fa_fwd().  q is [B, N, S, d], k and v are
+    [B, Nk, S, d] with Nk dividing N (Nk < N: grouped-query attention); any strides with a contiguous last
+    dimension are passed through (a [B, S, N, d] tensor is given as ``t.transpose(1, 2)``), any S >= 1.
     ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26)."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise ValueError("q, k, v must live on the GPU")
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise ValueError("q, k, v must share dtype float16 or bfloat16")
-    if q.shape != k.shape or q.shape != v.shape or q.dim() != 4:
-        raise ValueError("q, k, v must share shape [B, N, S, d]")
-    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
-        raise ValueError("q, k, v must be contiguous [B, N, S, d]")
+    if q.dim() != 4 or k.shape != v.shape or k.dim() != 4 or (q.shape[0], q.shape[2], q.shape[3]) != (
+            k.shape[0], k.shape[2], k.shape[3]) or k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0:
+        raise ValueError("q must be [B, N, S, d], k and v [B, Nk, S, d] with Nk dividing N")
+    if q.stride(3) != 1 or k.stride(3) != 1 or v.stride(3) != 1:
+        raise ValueError("the head dimension of q, k, v must be contiguous")
     B, N, S, d = q.shape
+    Nk = k.shape[1]
     if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
                                          and alibi_slopes.is_contiguous() and tuple(alibi_slopes.shape) == (N,)):
         raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
     if out is None:
-        out = torch.empty_like(q)
+        out = torch.empty_like(q)          # keeps q's strides
+    if out.shape != q.shape or out.dtype != q.dtype or out.stride(3) != 1:
+        raise ValueError("out must have q's shape and dtype and a contiguous head dimension")
     if return_lse and lse is None:
         lse = torch.empty((B, N, S), dtype=torch.float32, device=q.device)
     p = make_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                     lse.data_ptr() if return_lse else 0, softmax_scale, causal, window_left, window_right,
                     FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched,
-                    0 if alibi_slopes is None else alibi_slopes.data_ptr())
+                    0 if alibi_slopes is None else alibi_slopes.data_ptr(), 0 if Nk == N else Nk,
+                    *[None if t.is_contiguous() else tuple(t.stride()[:3]) for t in (q, k, v, out)])
     stream = torch.cuda.current_stream(q.device).cuda_stream
     st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
     if st != FA_OK:

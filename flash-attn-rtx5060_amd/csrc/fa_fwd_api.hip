@@ -17,7 +17,10 @@
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
-hipError_t fa_launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream);
+hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
+                                        hipStream_t stream);
+hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
+                                     hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -76,7 +79,8 @@ const char *fa_strerror(int status)
     case FA_ERR_NULL_POINTER: return "Q, K, V or O is NULL";
     case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FA_ERR_SEQLEN_MULTIPLE: return "seqlen must be a multiple of 128";
+    case FA_ERR_SEQLEN_MULTIPLE: return "reserved (seqlen no longer has to be a multiple of 128)";
+    case FA_ERR_LAYOUT: return "strides must be multiples of 8 elements (row strides at least head_dim), n_kv_heads must divide heads, pointers must be 16-byte aligned";
     case FA_ERR_UNSUPPORTED: return "dropout is not supported";
     case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
     case FA_ERR_SCALE: return "softmax_scale must be finite and positive";
@@ -154,12 +158,23 @@ int fa_fwd_validate(const fa_fwd_params *p)
     if (!p || !p->Q || !p->K || !p->V || !p->O) return FA_ERR_NULL_POINTER;
     if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
     if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
-    if (p->S % 128 != 0) return FA_ERR_SEQLEN_MULTIPLE;
     if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
     if (p->dropout_prob != 0.0f || p->states != nullptr) return FA_ERR_UNSUPPORTED;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
+    const void *ptrs[4] = {p->Q, p->K, p->V, p->O};
+    const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
+    for (int t = 0; t < 4; ++t) {
+        if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0) return FA_ERR_LAYOUT;
+        const long long *st = strides[t];
+        if (st[0] == 0 && st[1] == 0 && st[2] == 0) continue;       // contiguous
+        for (int k = 0; k < 3; ++k)
+            if (st[k] < 0 || st[k] % 8 != 0) return FA_ERR_LAYOUT;
+        if (st[2] < p->d) return FA_ERR_LAYOUT;
+        if (st[2] > (1LL << 24)) return FA_ERR_TOO_LARGE;           // per-lane byte offsets inside a tile are 32-bit
+    }
     return FA_OK;
 }
 
@@ -178,12 +193,34 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.H = p->N;
     a.BH = p->B * p->N;
     a.S = p->S;
+    // layout: contiguous [B,N,S,d] unless strides are given; K and V have n_kv_heads heads
+    a.Hk = p->n_kv_heads > 0 ? p->n_kv_heads : p->N;
+    bool general = a.Hk != p->N || p->S % 128 != 0;
+    {
+        const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
+        long long eff[4][3];
+        for (int t = 0; t < 4; ++t) {
+            const long long heads = (t == 1 || t == 2) ? a.Hk : p->N;
+            const long long dense[3] = {heads * p->S * p->d, (long long)p->S * p->d, p->d};
+            const long long *st = strides[t];
+            const bool given = st[0] != 0 || st[1] != 0 || st[2] != 0;
+            for (int k = 0; k < 3; ++k) {
+                eff[t][k] = given ? st[k] : dense[k];
+                if (eff[t][k] != dense[k]) general = true;
+            }
+        }
+        a.q_bs = eff[0][0]; a.q_hs = eff[0][1]; a.q_rs = (int)eff[0][2];
+        a.k_bs = eff[1][0]; a.k_hs = eff[1][1]; a.k_rs = (int)eff[1][2];
+        a.v_bs = eff[2][0]; a.v_hs = eff[2][1]; a.v_rs = (int)eff[2][2];
+        a.o_bs = eff[3][0]; a.o_hs = eff[3][1]; a.o_rs = (int)eff[3][2];
+    }
     const int waves = waves_for(p->B, p->N, p->S);
     const int block_rows = 32 * waves;
     a.n_qblocks = (p->S + block_rows - 1) / block_rows;
     fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
-    const int masked = (a.L < p->S || a.R < p->S) ? 1 : 0;
-    a.descending = masked;
+    // (a sequence that ends inside a 64-key tile needs the element mask on that tile, whatever the mask)
+    const int masked = (a.L < p->S || a.R < p->S || p->S % kBlockKeysHost != 0) ? 1 : 0;
+    a.descending = (a.L < p->S || a.R < p->S) ? 1 : 0;
     a.scale = p->softmax_scale;
     a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
     a.n_items = (long long)a.BH * a.n_qblocks;
@@ -209,7 +246,8 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         }
     }
     const int shape = waves == 8 ? 0 : 1;
-    hipError_t e = fa_launch_forward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
+    hipError_t e = (general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
+        a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
     return FA_OK;
 }

@@ -1,0 +1,740 @@
+// FlashAttention forward for gfx950 (MI355X), hand-written HIP.
+//
+// Role of the reference's forward_kernel<> (reference src/flash_forward.h:78-366)
+// with its helpers apply_softmax (src/softmax.h:9-86) and apply_mask
+// (src/mask.h:10-84), designed for CDNA4 instead of translated:
+//
+//  * Transposed formulation.  Each wave owns 32 query rows and computes
+//    S^T = K * Q^T with v_mfma_f32_32x32x16 (M = keys, N = queries), so a lane
+//    holds ONE query column and 16 key rows of every 32x32 block.  The online
+//    softmax reductions (softmax.h:19-41,69-78 use quad shuffles) are then
+//    in-register plus one v_permlane32_swap between the two half-waves.
+//  * The S^T accumulator layout is exactly the B-operand layout of the second
+//    contraction O^T = V^T * P^T, so P never leaves registers (the role of the
+//    C->A fragment repack at flash_forward.h:269-278).  O^T keeps the query on
+//    the lane as well, so the rescale factor is a per-lane scalar.
+//  * V^T operands come from row-major V tiles in LDS through
+//    ds_read_b64_tr_b16 (the role of ldmatrix.trans, include/utils.h:38-45).
+//  * K/V tiles go global -> LDS directly (global_load_lds_dwordx4, the role of
+//    the TMA loads at include/utils.h:86-99), XOR-swizzled at 16-byte
+//    granularity on the global-address side so that both the ds_read_b128
+//    K-operand pattern and the transposed V pattern are free of bank conflicts
+//    without padding (the reference tiles are unswizzled, utils.h:168).  Two or
+//    three LDS stages per tensor replace the mbarrier ring (flash_forward.h:95-111).
+//  * Software pipelining inside every wave: the matrix instructions of
+//    PV(tile-1) and QK(tile+1) are interleaved, a few vector instructions at a
+//    time, with the softmax of `tile`, so the matrix core stays busy while the
+//    wave's own exp/max/convert work issues in the gaps (the reference runs
+//    QK, softmax and PV back to back, flash_forward.h:193-315).
+//  * exp2 with scale*log2(e) folded into one FMA, the rescale of O done only
+//    when a row maximum has grown by more than 2^8 (the reference recomputes
+//    the factor 4*d/8 times per tile, flash_forward.h:296-299), the -inf
+//    guard the reference lacks (softmax.h:55,83).
+//  * Masks are evaluated per element only on tiles that straddle a mask edge,
+//    and tiles that are fully masked for a wave are skipped by that wave (the
+//    reference masks every tile, mask.h:10-84).
+//  * Work items (batch*head, query block) are either dispatched one per
+//    workgroup in longest-first order, or walked by a persistent grid of one
+//    workgroup per CU in a snake over the same list (Schedule<0,...>,
+//    flash_forward.h:22-65, walks it round-robin in natural order).
+#ifndef FA_FWD_KERNEL_IMPL_H
+#define FA_FWD_KERNEL_IMPL_H
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fa_kernel_args.h"
+#include "fa_sched.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kBlockKeys = 64;          // keys per K/V tile
+constexpr float kRescaleLog2 = 8.0f;    // rescale O only when a row max grew by > 2^8
+
+template <bool BF16> struct Num;
+template <> struct Num<false> {
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
+};
+template <> struct Num<true> {
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    }
+};
+
+// 16-byte-chunk swizzles.  A tile row holds CPR = D/8 chunks.
+// K is read with ds_read_b128 by 16 lanes holding 16 consecutive rows and one
+// logical chunk: those must land on 16 different 16-byte bank groups.
+template <int CPR> __device__ __forceinline__ int k_swz(int row) { return CPR == 16 ? (row & 15) : ((row >> 1) & 7); }
+// V is read with ds_read_b64_tr_b16: 32 lanes cover 4 consecutive rows x 4
+// consecutive chunks; the 4 rows must land on 4 different 64-byte bank groups.
+template <int CPR> __device__ __forceinline__ int v_swz(int row) { return CPR == 16 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+
+__device__ __forceinline__ float swap_halves(float x)
+{
+    // lane l <-> lane l^32
+    auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr)
+{
+    return *(const __attribute__((address_space(3))) u32x4 *)addr;
+}
+__device__ __forceinline__ u32x2 lds_read_tr(uint32_t addr)
+{
+    i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4 *)addr);
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// One wave-wide direct global->LDS load: lane l copies 16 bytes from base + voff (its own address) to
+// LDS byte lds + 16*l.  Written as inline assembly so that the compiler does not order every later LDS
+// read behind it with a vmcnt(0) wait; completion is waited for explicitly with s_waitcnt vmcnt + barrier.
+__device__ __forceinline__ void dma_16(const char *base, uint32_t voff, uint32_t lds)
+{
+    const uint64_t b = (uint64_t)base;     // wave-uniform by construction; say so, so that it lives in SGPRs
+    // (readfirstlane returns a signed int: go through uint32_t, or the low half would sign-extend)
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory");
+}
+__device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int V> struct IntC { static constexpr int value = V; };
+
+// ---------------------------------------------------------------------------
+// First rows of a causal head, in the reference's own arithmetic.
+//
+// A query that sees only a handful of keys can produce outputs as large as
+// the values themselves (|O| up to 4 and more at unit variance), where one
+// fp16 ulp is the whole tolerance.  There the dominant error of the reference
+// CPU verifier is its own rounding of every q*k and p*v product to the storage
+// type (reference src/main.cu:193,259): it is off from the exact result by up
+// to 3e-3 in those rows, and a kernel that accumulates exact products cannot
+// land on the same side.  For the first kFaithfulRows rows of every head (at
+// most that many visible keys under a causal mask) the workgroup therefore
+// recomputes the result with exactly the reference's sequence: product
+// rounded to the storage type, fp32 sums in index order, max-subtracted expf,
+// fp32 normalisation, p rounded to the storage type (main.cu:189-263).  It is
+// 32 x 32 scores and 32 x D outputs of scalar work per head.
+// ---------------------------------------------------------------------------
+constexpr int kFaithfulRows = 32;
+
+template <bool BF16> __device__ __forceinline__ float storage_to_f32(uint16_t h)
+{
+    if (BF16) return __builtin_bit_cast(float, (uint32_t)h << 16);
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+template <bool BF16> __device__ __forceinline__ uint16_t f32_to_storage(float x)
+{
+    if (BF16) return __builtin_bit_cast(uint16_t, (__bf16)x);
+    return __builtin_bit_cast(uint16_t, (_Float16)x);
+}
+// storage-type product of two storage-type values: the fp32 product is exact, one rounding to nearest even
+template <bool BF16> __device__ __forceinline__ float storage_product(float a, float b)
+{
+    return storage_to_f32<BF16>(f32_to_storage<BF16>(a * b));
+}
+
+template <bool BF16, int D>
+__device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
+                                    float *lse_h, int S, int L, float scale, float slope,
+                                    int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
+                                    float *sc /* LDS, 32*32 floats */)
+{
+    constexpr int R = kFaithfulRows;
+    const int rows = S < R ? S : R;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    // scores (main.cu:189-197), masked entries -inf (main.cu:210-229)
+    for (int idx = tid; idx < R * R; idx += nthr) {
+        const int i = idx / R, j = idx % R;
+        float s = -INFINITY;
+        if (i < rows && j <= i && i - j <= L) {
+            float sum = 0.0f;
+            for (int t = 0; t < D; ++t)
+                sum += storage_product<BF16>(storage_to_f32<BF16>(Qh[(size_t)i * q_rs + t]), storage_to_f32<BF16>(Kh[(size_t)j * k_rs + t]));
+            s = sum * scale;
+            // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
+            if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(i - j)));
+        }
+        sc[idx] = s;
+    }
+    __syncthreads();
+    // softmax of each row (main.cu:232-252), p rounded to the storage type (main.cu:259)
+    if (tid < rows) {
+        float *row = sc + tid * R;
+        float mx = -INFINITY;
+        for (int j = 0; j <= tid; ++j) mx = fmaxf(mx, row[j]);
+        float sum = 0.0f;
+        for (int j = 0; j <= tid; ++j) { row[j] = expf(row[j] - mx); sum += row[j]; }
+        for (int j = 0; j <= tid; ++j) row[j] = storage_to_f32<BF16>(f32_to_storage<BF16>(row[j] / sum));
+        if (lse_h != nullptr) lse_h[tid] = mx + logf(sum);
+    }
+    __syncthreads();
+    // weighted sum (main.cu:255-263), keys in ascending order; masked keys have p = 0 and add nothing
+    for (int idx = tid; idx < rows * D; idx += nthr) {
+        const int i = idx / D, t = idx % D;
+        const int lo = i - L > 0 ? i - L : 0;
+        float sum = 0.0f;
+        for (int j = lo; j <= i; ++j) sum += storage_product<BF16>(sc[i * R + j], storage_to_f32<BF16>(Vh[(size_t)j * v_rs + t]));
+        Oh[(size_t)i * o_rs + t] = f32_to_storage<BF16>(sum);
+    }
+    __syncthreads();
+}
+
+// ---------------------------------------------------------------------------
+// The kernel.  NW waves per workgroup, RB blocks of 32 query rows per wave,
+// NST LDS stages per tensor.  Every wave runs ONE instruction stream per key
+// tile; tiles are issued NST-1 iterations before their first use; one
+// workgroup barrier per tile.  With RB = 2 every K/V fragment read from LDS
+// feeds two matrix instructions, and the wave needs the whole 512-entry
+// register file of its SIMD (one wave per SIMD).
+// ---------------------------------------------------------------------------
+template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, int NW, int RB, int NST>
+__global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
+{
+    constexpr int WR = 32 * RB;                   // query rows per wave
+    constexpr int BR = WR * NW;                   // query rows per workgroup
+    constexpr int CPR = D / 8;
+    constexpr int ROWB = D * 2;
+    constexpr int TILEB = kBlockKeys * ROWB;
+    constexpr int INSTR = TILEB / 1024;
+    constexpr int IPW = INSTR / NW;               // direct-to-LDS instructions per wave per tile
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int NPV = 4 * DB;                   // V^T fragments per tile: (16-key slice, head-dim block)
+    constexpr int NQK = 2 * KS;                   // K fragments per tile: (head-dim slice, 32-key block)
+    constexpr int NF = NPV + NQK;                 // every fragment feeds RB matrix instructions
+    constexpr int PD = RB == 1 ? 6 : 3;           // LDS reads run this many fragments ahead
+    constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
+    constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
+    static_assert(INSTR % NW == 0, "tile must divide over the waves");
+    static_assert(NST >= 2 && NST <= 3 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
+    typedef Num<BF16> N;
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
+
+    // Work items.  Without a queue the grid is static: one workgroup per item (a single pass), or a resident
+    // grid that walks the longest-first list as a snake (pass 0 forwards, pass 1 backwards, ...), pairing
+    // long items with short ones.  With a queue, a resident grid takes items dynamically: a workgroup on XCD x
+    // takes list positions x, x+8, x+16, ... from that XCD's counter, so a head stays on one XCD's L2 and a
+    // workgroup that finishes early simply takes the next item -- the hardware dispatcher's longest-first
+    // greedy schedule without its workgroup launch gaps (about 10 us per item on this chip).
+    const int G = (int)gridDim.x;
+    unsigned xcd = 0;
+    if (a.queue != nullptr) {
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcd));
+        xcd &= 7u;
+    }
+    volatile unsigned *next_slot = reinterpret_cast<volatile unsigned *>(smem + 2 * NST * TILEB);
+    for (int pass = 0;; ++pass) {
+    long long item;
+    if (a.queue == nullptr) {
+        if ((long long)pass * G >= a.n_items) break;
+        item = (long long)pass * G + ((pass & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x);
+        if (item >= a.n_items) continue;
+    } else {
+        if (tid == 0) {
+            // own XCD's list first; when that is exhausted, help the others (this also makes the result
+            // independent of how the hardware spreads the workgroups over the XCDs)
+            unsigned found = 0xffffffffu;
+            for (unsigned xo = 0; xo < 8u && found == 0xffffffffu; ++xo) {
+                const unsigned xq = (xcd + xo) & 7u;
+                const long long cand = (long long)atomicAdd(&a.queue[xq], 1u) * 8 + xq;
+                if (cand < a.n_items) found = (unsigned)cand;
+            }
+            *next_slot = found;
+        }
+        __syncthreads();
+        // uniform by construction: say so, or everything derived from the item lives in vector registers
+        const unsigned taken = (unsigned)__builtin_amdgcn_readfirstlane((int)*next_slot);
+        __syncthreads();
+        if (taken == 0xffffffffu) break;
+        item = (long long)taken;
+    }
+    int bh, qblock;
+    fa_item_decode(item, a.BH, a.n_qblocks, a.descending, &bh, &qblock);
+    const int S = a.S;
+    // Contiguous [B,H,S,D] tensors, one K/V head per query head, S a multiple of 128: everything below is
+    // compile-time.  GENERAL: any strides (in elements, head dimension contiguous), query heads sharing K/V
+    // heads in groups of H/Hk, any S (rows past the end are read from row S-1 and never stored, keys past the
+    // end are masked like any other masked key).
+    const uint16_t *Qh, *Kh, *Vh;
+    uint16_t *Oh;
+    if (GENERAL) {
+        const int bi = bh / a.H, hi = bh - bi * a.H, hk = hi / (a.H / a.Hk);
+        Qh = a.Q + (size_t)bi * a.q_bs + (size_t)hi * a.q_hs;
+        Kh = a.K + (size_t)bi * a.k_bs + (size_t)hk * a.k_hs;
+        Vh = a.V + (size_t)bi * a.v_bs + (size_t)hk * a.v_hs;
+        Oh = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs;
+    } else {
+        const size_t head_off = (size_t)bh * S * D;
+        Qh = a.Q + head_off; Kh = a.K + head_off; Vh = a.V + head_off;
+        Oh = a.O + head_off;
+    }
+    const int q_rs = GENERAL ? a.q_rs : D, k_rs = GENERAL ? a.k_rs : D, v_rs = GENERAL ? a.v_rs : D, o_rs = GENERAL ? a.o_rs : D;
+
+    const int q0 = qblock * BR;
+    const int qw = q0 + wave * WR;          // first query row of this wave
+    const int my_q = qw + l32;              // query row of row block 0 on this lane; block b adds 32*b
+    const bool wave_live = qw < S;          // (not GENERAL: S is a multiple of 128, a live wave has all its rows)
+
+    // Q^T fragments: B operand, lane = (query l32, head-dim slice 8*half..+7 of each 16)
+    u32x4 qf[RB][KS];
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(
+                                       Qh + (size_t)((GENERAL && my_q + 32 * b >= S) ? S - 1 : my_q + 32 * b) * q_rs + 16 * s + 8 * half)
+                                 : u32x4{0, 0, 0, 0};
+
+    const int rows_in_block = S - q0 < BR ? S - q0 : BR;
+    int t0, t1;                 // key tiles visited by the workgroup
+    fa_tile_range(S, kBlockKeys, a.L, a.R, q0, rows_in_block, &t0, &t1);
+    int my_lo = 1, my_hi = 0;   // key tiles with at least one visible pair for this wave (contiguous)
+    if (wave_live) fa_tile_range(S, kBlockKeys, a.L, a.R, qw, WR, &my_lo, &my_hi);
+
+    // per-lane LDS read addresses for stage 0; stage, key block and key slice are immediates
+    uint32_t koff[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+        koff[s] = lds0 + (uint32_t)(l32 * ROWB + (((2 * s + half) ^ k_swz<CPR>(l32)) << 4));
+    uint32_t voff[DB];
+    {
+        const int row0 = 4 * half + (l16 >> 2);
+        const int dq = (l32 >> 4), c4 = l16 & 3;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const int c = 4 * db + 2 * dq + (c4 >> 1);
+            voff[db] = lds0 + LDS_V + (uint32_t)(row0 * ROWB + ((c ^ v_swz<CPR>(row0)) << 4) + ((c4 & 1) << 3));
+        }
+    }
+    // direct global -> LDS tile loads: wave w issues instructions w, w+NW, ... of the tile; instruction n
+    // fills LDS bytes [n*1024, n*1024+1024) linearly, lane l supplying the swizzled source chunk.
+    uint32_t gk[IPW], gv[IPW];
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) {
+        const int P = (i * NW + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
+        gk[i] = (uint32_t)(row * (k_rs * 2) + ((pos ^ k_swz<CPR>(row)) << 4));
+        gv[i] = (uint32_t)(row * (v_rs * 2) + ((pos ^ v_swz<CPR>(row)) << 4));
+    }
+    // (GENERAL: the rows of the last tile that lie past the end of the sequence are fetched from row S-1;
+    // they land in their own LDS rows and are masked)
+    auto ragged_source = [&](int tile, int i, int rs, bool is_k) __attribute__((always_inline)) {
+        const int P = (i * NW + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
+        const int last = S - 1 - tile * kBlockKeys, src_row = row < last ? row : last;
+        return (uint32_t)(src_row * (rs * 2) + ((pos ^ (is_k ? k_swz<CPR>(row) : v_swz<CPR>(row))) << 4));
+    };
+    auto issue_k = [&](int tile, int stage) __attribute__((always_inline)) {
+        const char *src = reinterpret_cast<const char *>(Kh) + (size_t)tile * (kBlockKeys * 2) * k_rs;
+        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > S;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i)
+            dma_16(src, ragged ? ragged_source(tile, i, k_rs, true) : gk[i], lds0 + stage * TILEB + (i * NW + wave) * 1024);
+    };
+    auto issue_v = [&](int tile, int stage) __attribute__((always_inline)) {
+        const char *src = reinterpret_cast<const char *>(Vh) + (size_t)tile * (kBlockKeys * 2) * v_rs;
+        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > S;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i)
+            dma_16(src, ragged ? ragged_source(tile, i, v_rs, false) : gv[i], lds0 + LDS_V + stage * TILEB + (i * NW + wave) * 1024);
+    };
+    // skip / edge / free classification of a key tile for this wave (GENERAL: a tile that reaches past the
+    // end of the sequence is an edge tile)
+    auto tile_class = [&](int tile) __attribute__((always_inline)) {
+        int cls = fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile);
+        if (GENERAL && cls == 2 && (tile + 1) * kBlockKeys > S) cls = 1;
+        return cls;
+    };
+
+    f32x16 o[RB][DB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][db][r] = 0.0f;
+    float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
+#pragma unroll
+    for (int b = 0; b < RB; ++b) { m_run[b] = -INFINITY; l_a[b] = 0.0f; l_b[b] = 0.0f; }
+    // Without ALiBi the tile scores stay raw dot products and the softmax scale is folded into the exponent
+    // (exp2(s*c - m*c)).  With ALiBi a tile is first rewritten in place to log2 units with the bias applied,
+    // s*c - slope*log2(e)*|i-j| (mask.h:21-26 subtracts slope*|i-j| from the scaled score), so maxima, the
+    // reference point and the exponent work on those values with a factor of one.
+    const float c = a.scale_log2e;
+    const float cs = ALIBI ? 1.0f : c;
+    const float slope = ALIBI ? a.alibi[bh % a.H] : 0.0f;
+    const float slope_l2 = slope * 1.44269504088896340736f;
+    const float thresh = kRescaleLog2 / cs;
+    uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
+    f32x16 sx[RB][2];           // S^T of the tile whose softmax comes next: [key block 0 / 1]
+
+    auto read_v = [&](uint32_t vs, int n) __attribute__((always_inline)) {
+        const int t2 = n / DB, db = n % DB;
+        const u32x2 lo = lds_read_tr(voff[db] + vs + (16 * t2) * ROWB);
+        const u32x2 hi = lds_read_tr(voff[db] + vs + (16 * t2 + 8) * ROWB);
+        return u32x4{lo[0], lo[1], hi[0], hi[1]};
+    };
+    auto read_k = [&](uint32_t ks, int n) __attribute__((always_inline)) {
+        return lds_read_b128(koff[n >> 1] + ks + (n & 1) * 32 * ROWB);
+    };
+    auto apply_mask = [&](int tile) __attribute__((always_inline)) {
+        const int kb0 = tile * kBlockKeys + 4 * half;
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const int q = my_q + 32 * b;
+            // last visible key of this query (GENERAL: the sequence may end inside the tile)
+            const int j_hi = (GENERAL && q + a.R > S - 1) ? S - 1 : q + a.R;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
+                const int j1 = j0 + 32;
+                if (j0 > j_hi || j0 < q - a.L) sx[b][0][r] = -INFINITY;
+                if (j1 > j_hi || j1 < q - a.L) sx[b][1][r] = -INFINITY;
+            }
+        }
+    };
+    auto apply_alibi = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            // signed distance of this lane's query to the lane's first key of the tile: exact in fp32
+            const float base = (float)(my_q + 32 * b - (tile * kBlockKeys + 4 * half));
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float k0 = (float)(8 * (r >> 2) + (r & 3));
+                sx[b][0][r] = __builtin_fmaf(__builtin_fabsf(base - k0), -slope_l2, sx[b][0][r] * c);
+                sx[b][1][r] = __builtin_fmaf(__builtin_fabsf(base - (k0 + 32.0f)), -slope_l2, sx[b][1][r] * c);
+            }
+        }
+    };
+    auto row_max = [&](int b) __attribute__((always_inline)) {
+        float mx = fmaxf(sx[b][0][0], sx[b][1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, sx[b][0][r]), sx[b][1][r]);
+        return fmaxf(mx, swap_halves(mx));
+    };
+    // the decision to move the reference point of row block b; returns the factor by which everything
+    // accumulated so far has to be multiplied (1 when the reference point stays)
+    auto new_reference = [&](int b, float mx, bool &moved) __attribute__((always_inline)) {
+        float alpha = 1.0f;
+        const bool grow = mx > m_run[b] + thresh;   // -inf + thresh = -inf: a first finite max always grows
+        moved = __builtin_amdgcn_ballot_w64(grow) != 0;
+        if (moved) {
+            const float m_new = grow ? mx : m_run[b];
+            alpha = (m_run[b] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run[b] - m_new) * cs);
+            l_a[b] *= alpha;
+            l_b[b] *= alpha;
+            m_run[b] = m_new;
+        }
+        return alpha;
+    };
+    auto scale_o = [&](int b, float alpha) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][db][r] *= alpha;
+    };
+    auto p_operand = [&](int b, int t2) __attribute__((always_inline)) {
+        return u32x4{pk[b][4 * t2], pk[b][4 * t2 + 1], pk[b][4 * t2 + 2], pk[b][4 * t2 + 3]};
+    };
+
+    // ---- plain (not interleaved) pieces, used while the pipeline fills and drains
+    // (the scheduling barriers keep register pressure low here: without them the compiler hoists every
+    // LDS read of the unrolled loop to the top and spills)
+    auto pv_plain = [&](int vstage) __attribute__((always_inline)) {
+        const uint32_t vs = vstage * TILEB;
+        u32x4 fr[NPV];
+        fr[0] = read_v(vs, 0);
+        fr[1] = read_v(vs, 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int n = 0; n < NPV; ++n) {
+            if (n + 2 < NPV) fr[n + 2] = read_v(vs, n + 2);
+            const int t2 = n / DB, db = n % DB;
+#pragma unroll
+            for (int b = 0; b < RB; ++b) o[b][db] = N::mfma(fr[n], p_operand(b, t2), o[b][db]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto qk_plain = [&](int kstage) __attribute__((always_inline)) {
+        const uint32_t ks = kstage * TILEB;
+        u32x4 fr[NQK];
+        fr[0] = read_k(ks, 0);
+        fr[1] = read_k(ks, 1);
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sx[b][0][r] = 0.0f; sx[b][1][r] = 0.0f; }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int n = 0; n < NQK; ++n) {
+            if (n + 2 < NQK) fr[n + 2] = read_k(ks, n + 2);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) sx[b][n & 1] = N::mfma(fr[n], qf[b][n >> 1], sx[b][n & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
+        if (ALIBI) apply_alibi(tile);
+        if (MASKED && tile_class(tile) == 1) apply_mask(tile);
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            bool moved;
+            const float alpha = new_reference(b, row_max(b), moved);
+            if (moved) scale_o(b, alpha);
+            const float mc = (m_run[b] == -INFINITY) ? 0.0f : m_run[b] * cs;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], cs, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i + 1], cs, -mc));
+                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], cs, -mc));
+                const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], cs, -mc));
+                l_a[b] += e0; l_b[b] += e1; l_a[b] += e2; l_b[b] += e3;
+                pk[b][i] = N::pack2(e0, e1);
+                pk[b][8 + i] = N::pack2(e2, e3);
+            }
+        }
+    };
+
+    // ---- the steady-state iteration: PV(tile-1) from V stage VST, softmax(tile), QK(tile+1) from K stage KST
+    auto steady = [&](auto KST, auto VST, int tile) __attribute__((always_inline)) {
+        constexpr uint32_t ks = decltype(KST)::value * TILEB;
+        constexpr uint32_t vs = decltype(VST)::value * TILEB;
+        u32x4 fr[NF];                              // operand fragments, in the order they are consumed
+        auto fetch = [&](int n) __attribute__((always_inline)) {
+            if (n < NPV) fr[n] = read_v(vs, n);
+            else fr[n] = read_k(ks, n - NPV);
+        };
+#pragma unroll
+        for (int n = 0; n < PD; ++n) fetch(n);
+        // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
+        if (ALIBI) apply_alibi(tile);
+        if (MASKED && tile_class(tile) == 1) apply_mask(tile);
+        bool moved[RB];
+        float alpha[RB], nmc[RB];
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            alpha[b] = new_reference(b, row_max(b), moved[b]);
+            nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * cs;
+        }
+        uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
+        f32x16 nx[RB][2];                          // S^T(tile+1)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < NF; ++g) {
+            if (g + PD < NF) fetch(g + PD);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) {
+                if (g < NPV) {
+                    const int t2 = g / DB, db = g % DB;
+                    o[b][db] = N::mfma(fr[g], p_operand(b, t2), o[b][db]);
+                } else {
+                    const int n = g - NPV;
+                    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n < 2 ? zero : nx[b][n & 1]);
+                }
+                // softmax work riding along: the 16*RB element pairs of this tile spread over the NF*RB matrix
+                // instructions, row block 0 first (its registers are free again when S^T(tile+1) is born)
+                constexpr int PAIRS = 16 * RB, SLOTS = NF * RB;
+                const int slot = g * RB + b;
+                const int p_begin = (slot * PAIRS) / SLOTS, p_end = ((slot + 1) * PAIRS) / SLOTS;
+#pragma unroll
+                for (int pi = p_begin; pi < p_end; ++pi) {
+                    // pair e of row block pb: elements (2e, 2e+1) of key block 0 for e < 8, of key block 1 for
+                    // e >= 8.  The two empty asm statements pin the arithmetic between the surrounding matrix
+                    // instructions (without them the compiler sinks all of it to the end of the iteration);
+                    // the first goes through the subtrahend, which stays in one register, so it costs no move.
+                    const int pb = pi / 16, e = pi % 16;
+                    const float x0 = e < 8 ? sx[pb][0][2 * e] : sx[pb][1][2 * (e - 8)];
+                    const float x1 = e < 8 ? sx[pb][0][2 * e + 1] : sx[pb][1][2 * (e - 8) + 1];
+                    asm volatile("" : "+v"(nmc[pb]));
+                    const float e0 = __builtin_amdgcn_exp2f(ALIBI ? x0 + nmc[pb] : __builtin_fmaf(x0, c, nmc[pb]));
+                    const float e1 = __builtin_amdgcn_exp2f(ALIBI ? x1 + nmc[pb] : __builtin_fmaf(x1, c, nmc[pb]));
+                    l_a[pb] += e0;
+                    l_b[pb] += e1;
+                    uint32_t packed = N::pack2(e0, e1);
+                    asm volatile("" : "+v"(packed), "+v"(l_a[pb]), "+v"(l_b[pb]));
+                    pn[pb][e] = packed;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            if (moved[b]) scale_o(b, alpha[b]);    // rare; PV(tile-1) has been issued in full by now
+#pragma unroll
+            for (int i = 0; i < 16; ++i) pk[b][i] = pn[b][i];
+            sx[b][0] = nx[b][0];
+            sx[b][1] = nx[b][1];
+        }
+    };
+
+    // ---- prologue: K(t0) .. K(t0+LA-1) resident before the first iteration
+    issue_k(t0, 0);
+    if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
+    wait_vm<0>();
+    // Q has landed too (vmcnt is 0).  Touching the fragments here lets the compiler see that, so that it places
+    // no vmcnt wait of its own inside the loop, where it would also wait for the asynchronous tile loads.
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[b][s]));
+    phase_barrier();
+
+    // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST
+    // of its tensor, so the iteration reads K stage j % NST and V stage (j - 2) % NST; it issues the loads of
+    // K(i+1+LA) and V(i-1+LA), which overwrite tiles whose last readers ran one iteration ago.
+    // Every wave executes every iteration (one barrier each); a wave whose own tile range does not cover all
+    // three pieces runs the plain pieces it has, the others run the interleaved body.  The two kinds live in
+    // separate loops: merging them under one branch makes the register allocator spill.
+    auto finish_iteration = [&](bool full_issue) __attribute__((always_inline)) {
+        // what the next iteration reads must have landed; with three stages that was issued one iteration
+        // ago, so the loads issued just now may stay in flight
+        if (NST == 3 && full_issue) wait_vm<2 * IPW>();
+        else wait_vm<0>();
+        phase_barrier();
+    };
+    auto generic_iteration = [&](int i, int j3) __attribute__((always_inline)) {
+        const int tk = i + 1 + LA, tv = i - 1 + LA;
+        const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
+        const int jm1 = j3 == 0 ? NST - 1 : j3 - 1, jm2 = jm1 == 0 ? NST - 1 : jm1 - 1, jm3 = jm2 == 0 ? NST - 1 : jm2 - 1;
+        if (more_k) issue_k(tk, jm1);              // (j + LA) % NST == (j - 1) % NST
+        if (more_v) issue_v(tv, jm3);              // (j - 2 + LA) % NST == (j - 3) % NST
+        if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(jm2);
+        if (my_lo <= i && i <= my_hi) softmax_plain(i);
+        if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3);
+        finish_iteration(more_k && more_v);
+    };
+    auto steady_iteration = [&](auto J3, int i) __attribute__((always_inline)) {
+        constexpr int j3 = decltype(J3)::value;
+        constexpr int jm1 = (j3 + NST - 1) % NST, jm2 = (j3 + 2 * NST - 2) % NST, jm3 = (j3 + 3 * NST - 3) % NST;
+        const int tk = i + 1 + LA, tv = i - 1 + LA;
+        const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
+        if (more_k) issue_k(tk, jm1);
+        if (more_v) issue_v(tv, jm3);
+        steady(IntC<j3>{}, IntC<jm2>{}, i);
+        finish_iteration(more_k && more_v);
+    };
+    int i = t0 - 1, j3 = 0;
+    for (; i <= t1 + 1; ++i) {            // fill: until NST consecutive iterations are steady and the stage is 0
+        if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
+        generic_iteration(i, j3);
+        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+    }
+    for (; i >= my_lo + 1 && i + NST - 1 <= my_hi - 1 && i <= t1 + 1; i += NST) {
+        steady_iteration(IntC<0>{}, i);
+        steady_iteration(IntC<1>{}, i + 1);
+        if (NST == 3) steady_iteration(IntC<2 % NST>{}, i + 2);
+    }
+    for (j3 = 0; i <= t1 + 1; ++i) {      // drain
+        generic_iteration(i, j3);
+        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+    }
+
+    // rows 0..31 of a causal head are written by faithful_first_rows below instead
+    const bool faithful = MASKED && a.R == 0 && q0 == 0;
+    if (wave_live) {
+        // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides)
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            if (faithful && wave == 0 && b == 0) continue;
+            const int q = my_q + 32 * b;
+            if (GENERAL && q >= S) continue;       // a row past the end of the sequence
+            const float l_half = l_a[b] + l_b[b];
+            const float l_tot = l_half + swap_halves(l_half);
+            const float inv = 1.0f / l_tot;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
+                    w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2 *>(Oh + (size_t)q * o_rs + 32 * db + 8 * g + 4 * half) = w;
+                }
+            if (a.lse != nullptr && half == 0)
+                a.lse[(size_t)bh * S + q] = m_run[b] * (ALIBI ? 0.69314718055994530942f : a.scale) + __builtin_logf(l_tot);
+        }
+    }
+    if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
+        faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
+                                     slope, q_rs, k_rs, v_rs, o_rs, reinterpret_cast<float *>(smem));
+    }   // next work item
+    // the last workgroup to leave rewinds the queue for the next launch that uses it
+    if (a.queue != nullptr && tid == 0) {
+        __threadfence();
+        if (atomicAdd(&a.queue[8], 1u) == (unsigned)G - 1u) {
+#pragma unroll
+            for (int x = 0; x < 9; ++x) a.queue[x] = 0u;
+        }
+    }
+}
+
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, int NW, int RB, int NST>
+hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
+{
+    constexpr int TILEB = kBlockKeys * D * 2;
+    const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, NW, RB, NST>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
+    return hipGetLastError();
+}
+
+
+// shape 0: 8 waves x 32 rows = 256 query rows per workgroup, three LDS stages, one workgroup per CU.
+// shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
+// (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
+// answers it with about 500 AGPR<->VGPR moves per tile.)
+template <bool GENERAL>
+hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
+{
+    const int alibi = a.alibi != nullptr;
+#define FA_CASE(BF, DD, MK, AL) \
+    if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, 8, 1, 3>(a, grid, stream); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, 4, 1, 2>(a, grid, stream); \
+    }
+#define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
+    FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)
+#undef FA_CASES
+#undef FA_CASE
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+#endif

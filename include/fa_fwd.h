@@ -8,8 +8,9 @@
  * opaque `void *` (a hipStream_t, NULL = the default stream).
  *
  * Tensors are contiguous [B, N, S, d] 16-bit (fp16 or bf16), exactly as the
- * reference lays them out (reference src/main.cu:182, flash_forward.h:378-381);
- * the logsumexp output is fp32 [B, N, S].
+ * reference lays them out (reference src/main.cu:182, flash_forward.h:378-381),
+ * unless fa_fwd_params gives strides; the logsumexp output is fp32 [B, N, S].
+ * d is 64 or 128; S is any positive length (the reference needs S % 128 == 0).
  */
 #ifndef FA_FWD_H
 #define FA_FWD_H
@@ -27,13 +28,16 @@ enum {
     FA_ERR_NULL_POINTER = -1,      /* Q, K, V or O is NULL                                  */
     FA_ERR_BAD_SHAPE = -2,         /* B, N or S is not positive                              */
     FA_ERR_HEAD_DIM = -3,          /* d not in {64, 128}: reference throws, flash_forward.h:587 */
-    FA_ERR_SEQLEN_MULTIPLE = -4,   /* S % 128 != 0: reference assumes it silently, :134,637  */
+    FA_ERR_SEQLEN_MULTIPLE = -4,   /* reserved (was: S % 128 != 0, which the reference assumes silently,
+                                      :134,637); any S >= 1 is accepted now                 */
     FA_ERR_UNSUPPORTED = -5,       /* dropout requested                                      */
     FA_ERR_DTYPE = -6,             /* dtype is neither FA_DTYPE_F16 nor FA_DTYPE_BF16        */
     FA_ERR_SCALE = -7,             /* softmax_scale is not a finite positive number          */
     FA_ERR_DEVICE = -8,            /* a HIP runtime call failed; see fa_last_device_error()  */
     FA_ERR_NO_DEVICE = -9,         /* no gfx950 device is visible                            */
-    FA_ERR_TOO_LARGE = -10         /* B*N*S*d or the work-item count overflows the kernel's index range */
+    FA_ERR_TOO_LARGE = -10,        /* B*N*S*d or the work-item count overflows the kernel's index range */
+    FA_ERR_LAYOUT = -11            /* a stride is not a multiple of 8 elements or too small, n_kv_heads does
+                                      not divide N, or a tensor pointer is not 16-byte aligned */
 };
 
 enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
@@ -80,6 +84,15 @@ typedef struct fa_fwd_params {
     int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                 */
     int is_causal;            /* keys with j > i are masked (mask.h:27-38)                    */
     int sched;                /* FA_SCHED_*                                                   */
+    /* --- layouts beyond the reference's contiguous [B,N,S,d] (main.cu:182); all zero = that layout --- */
+    int n_kv_heads;           /* K/V heads per batch entry, 0 = N.  Must divide N: query head h reads K/V
+                                 head h / (N / n_kv_heads) (grouped-query / multi-query attention)      */
+    long long q_strides[3];   /* batch, head and row (sequence position) strides of Q in elements; the
+                                 head dimension is contiguous.  {0,0,0} = contiguous [B,N,S,d];
+                                 a [B,S,N,d] tensor is {S*N*d, d, N*d}                                  */
+    long long k_strides[3];   /* same for K ({0,0,0} = contiguous [B,n_kv_heads,S,d])                   */
+    long long v_strides[3];
+    long long o_strides[3];   /* same for O ({0,0,0} = contiguous [B,N,S,d]); L is always [B,N,S]       */
 } fa_fwd_params;
 
 /* Checks a parameter block without touching any device.  Returns FA_OK or the

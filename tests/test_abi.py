@@ -29,8 +29,22 @@ def test_struct_layout_matches_header(fa):
     text = open(os.path.join(REPO, "include", "fa_fwd.h")).read()
     body = re.search(r"typedef struct fa_fwd_params \{(.*?)\} fa_fwd_params;", text, flags=re.S).group(1)
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
-    fields = [re.search(r"(\w+)\s*;", line).group(1) for line in body.splitlines() if ";" in line]
+    fields = [re.search(r"(\w+)\s*(\[\d+\])?\s*;", line).group(1) for line in body.splitlines() if ";" in line]
     assert fields == [f[0] for f in fa.FaFwdParams._fields_]
+    # size and the offset of the last field as the C compiler lays the struct out
+    import subprocess
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "layout.c")
+        with open(src, "w") as f:
+            f.write('#include <stdio.h>\n#include <stddef.h>\n#include "fa_fwd.h"\n'
+                    'int main(void){printf("%zu %zu %zu\\n", sizeof(fa_fwd_params), offsetof(fa_fwd_params, o_strides),'
+                    ' offsetof(fa_fwd_params, dtype));return 0;}\n')
+        exe = os.path.join(tmp, "layout")
+        subprocess.run(["gcc", "-I", os.path.join(REPO, "include"), src, "-o", exe], check=True)
+        size, off_last, off_dtype = (int(x) for x in subprocess.run([exe], check=True, stdout=subprocess.PIPE, text=True).stdout.split())
+    assert size == ctypes.sizeof(fa.FaFwdParams)
+    assert off_last == fa.FaFwdParams.o_strides.offset and off_dtype == fa.FaFwdParams.dtype.offset
     # the first twenty are mykernelParamType's, in its order (include/utils.h:143-165)
     assert fields[:20] == ["Q", "K", "V", "O", "L", "M", "B", "N", "S", "d", "Tr", "Tc", "softmax_scale", "dropout_prob",
                            "seed", "states", "window_size_left", "window_size_right", "alibi_slopes_ptr", "split_num"]
@@ -62,8 +76,8 @@ def test_validate_status_codes(fa):
     assert status(S=0) == fa.FA_ERR_BAD_SHAPE
     for d in (0, 32, 96, 256):
         assert status(d=d, softmax_scale=0.1) == fa.FA_ERR_HEAD_DIM            # the reference throws, flash_forward.h:587-589
-    for S in (64, 100, 2048 + 64):
-        assert status(S=S) == fa.FA_ERR_SEQLEN_MULTIPLE     # the reference silently assumes it
+    for S in (1, 64, 100, 2048 + 64):
+        assert status(S=S) == fa.FA_OK                      # any length (the reference silently assumes S % 128 == 0)
     assert status(dtype=2) == fa.FA_ERR_DTYPE
     assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE
     assert status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE
@@ -72,6 +86,17 @@ def test_validate_status_codes(fa):
     assert status_raw(dict(states=0x10)) == fa.FA_ERR_UNSUPPORTED
     assert status_raw(dict(alibi_slopes_ptr=0x10)) == fa.FA_OK               # ALiBi slopes are accepted
     assert status(B=70000, N=70000, S=128) == fa.FA_ERR_TOO_LARGE
+    # layouts: K/V heads must divide the query heads, strides are multiples of 8 elements with a row stride of
+    # at least the head dimension, pointers are 16-byte aligned
+    assert status(n_kv_heads=2) == fa.FA_OK and status(n_kv_heads=8) == fa.FA_OK
+    assert status(n_kv_heads=3) == fa.FA_ERR_LAYOUT and status(n_kv_heads=-1) == fa.FA_ERR_LAYOUT
+    bshd = (2048 * 8 * 64, 64, 8 * 64)
+    assert status(q_strides=bshd, k_strides=bshd, v_strides=bshd, o_strides=bshd) == fa.FA_OK
+    assert status(q_strides=(2048 * 8 * 64, 64, 8 * 64 + 4)) == fa.FA_ERR_LAYOUT
+    assert status(k_strides=(2048 * 8 * 64, 64, 32)) == fa.FA_ERR_LAYOUT
+    assert status(v_strides=(-8, 64, 512)) == fa.FA_ERR_LAYOUT
+    assert status(o_strides=(0, 0, 1 << 25)) == fa.FA_ERR_TOO_LARGE
+    assert status(q_ptr=0x1008) == fa.FA_ERR_LAYOUT
     # fa_fwd itself refuses the same blocks before touching any device
     p = fa.make_params(**dict(ok, d=96))
     assert L.fa_fwd(ctypes.byref(p), None) == fa.FA_ERR_HEAD_DIM
@@ -93,11 +118,11 @@ def test_reference_entry_point_rejects_unsupported_flags(fa):
 def test_strerror_covers_every_status(fa):
     L = fa.lib()
     seen = set()
-    for st in range(0, -11, -1):
+    for st in range(0, -12, -1):
         msg = L.fa_strerror(st).decode()
         assert msg and msg != "unknown status"
         seen.add(msg)
-    assert len(seen) == 11
+    assert len(seen) == 12
     assert L.fa_strerror(-99).decode() == "unknown status"
 
 
