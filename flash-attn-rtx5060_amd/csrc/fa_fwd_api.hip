@@ -230,15 +230,21 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     // workgroups that walk the list themselves.
     long long grid = a.n_items;
     a.queue = nullptr;
-    const int sched = p->sched == FA_SCHED_AUTO ? FA_SCHED_QUEUE : p->sched;
+    int cus = kComputeUnits;
+    {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    }
+    const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
+    // FA_SCHED_AUTO: with at most one item per resident workgroup there is nothing to schedule (and the
+    // queue's counter round trips, 2.3 us each, would double the run time of a 7 us problem); with at most
+    // two, the fixed snake pairs every long item with a short one; beyond that the work queue balances best.
+    // Measured: c1 9.5 / 9.5 / 5.8 TFLOP/s (dispatch / snake / queue), c2 431 / 516 / 434, c3 995 / - / 1012.
+    int sched = p->sched;
+    if (sched == FA_SCHED_AUTO)
+        sched = a.n_items <= resident ? FA_SCHED_DISPATCH : a.n_items <= 2 * resident ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
     if (sched == FA_SCHED_PERSISTENT || sched == FA_SCHED_QUEUE) {
-        int cus = kComputeUnits;
-        int dev = 0;
-        if (hipGetDevice(&dev) == hipSuccess) {
-            int n = 0;
-            if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
-        }
-        const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
         if (grid > resident) grid = resident;
         if (sched == FA_SCHED_QUEUE) {
             hipError_t qe = work_queue_for_launch(&a.queue);
