@@ -46,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_validate", "fa_fwd", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
+    "fa_dropout_threshold", "fa_dropout_keep",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
     "fa_event_elapsed_ms", "fa_event_destroy",
@@ -115,6 +116,8 @@ def lib():
         L.fa_count_pairs.argtypes = [ctypes.c_int] * 4
         L.fa_algorithmic_flops.restype = ctypes.c_double
         L.fa_algorithmic_flops.argtypes = [ctypes.c_int] * 7
+        L.fa_dropout_threshold.argtypes = [ctypes.c_float]
+        L.fa_dropout_keep.argtypes = [ctypes.c_ulonglong, ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -145,11 +148,12 @@ def host_lib():
 
 def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
                 window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0,
-                n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None):
+                n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None, dropout_prob=0.0, seed=0):
     """A filled fa_fwd_params.  Strides are (batch, head, row) in elements, None = contiguous [B,N,S,d]."""
     p = FaFwdParams()
     p.alibi_slopes_ptr = alibi_ptr or None
     p.n_kv_heads = n_kv_heads
+    p.dropout_prob, p.seed = dropout_prob, seed
     for name, st in (("q_strides", q_strides), ("k_strides", k_strides), ("v_strides", v_strides), ("o_strides", o_strides)):
         if st is not None:
             setattr(p, name, (ctypes.c_longlong * 3)(*st))
@@ -162,7 +166,8 @@ def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softm
 
 
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                            return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None):
+                            return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None,
+                            dropout_prob=0.0, seed=0):
     """O, LSE = attention(q, k, v) on the GPU through fa_fwd().  q is [B, N, S, d], k and v are
     [B, Nk, S, d] with Nk dividing N (Nk < N: grouped-query attention); any strides with a contiguous last
     dimension are passed through (a [B, S, N, d] tensor is given as ``t.transpose(1, 2)``), any S >= 1.
@@ -192,7 +197,8 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
                     lse.data_ptr() if return_lse else 0, softmax_scale, causal, window_left, window_right,
                     FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched,
                     0 if alibi_slopes is None else alibi_slopes.data_ptr(), 0 if Nk == N else Nk,
-                    *[None if t.is_contiguous() else tuple(t.stride()[:3]) for t in (q, k, v, out)])
+                    *[None if t.is_contiguous() else tuple(t.stride()[:3]) for t in (q, k, v, out)],
+                    dropout_prob=dropout_prob, seed=seed)
     stream = torch.cuda.current_stream(q.device).cuda_stream
     st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
     if st != FA_OK:

@@ -21,6 +21,8 @@ hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, 
                                         hipStream_t stream);
 hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
+hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
+                                     hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -81,7 +83,7 @@ const char *fa_strerror(int status)
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
     case FA_ERR_SEQLEN_MULTIPLE: return "reserved (seqlen no longer has to be a multiple of 128)";
     case FA_ERR_LAYOUT: return "strides must be multiples of 8 elements (row strides at least head_dim), n_kv_heads must divide heads, pointers must be 16-byte aligned";
-    case FA_ERR_UNSUPPORTED: return "dropout is not supported";
+    case FA_ERR_UNSUPPORTED: return "dropout_prob must be at least 0 and below 1";
     case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
     case FA_ERR_SCALE: return "softmax_scale must be finite and positive";
     case FA_ERR_DEVICE: return "HIP runtime error";
@@ -153,13 +155,36 @@ double fa_algorithmic_flops(int B, int N, int S, int d, int is_causal, int windo
     return 4.0 * (double)B * (double)N * (double)d * (double)fa_count_pairs(S, is_causal, window_left, window_right);
 }
 
+int fa_dropout_threshold(float dropout_prob)
+{
+    if (!(dropout_prob > 0.0f)) return 0;
+    const long t = lrintf(dropout_prob * 256.0f);
+    return t > 255 ? 255 : (int)t;
+}
+
+int fa_dropout_keep(unsigned long long seed, long long bh, int i, int j, int threshold)
+{
+    // One Philox4x32-10 block per (query, 32-key block, (j / 4) % 2): sixteen bytes for sixteen keys.
+    uint32_t c0 = (uint32_t)(2 * (j >> 5) + ((j >> 2) & 1)), c1 = (uint32_t)i, c2 = (uint32_t)bh, c3 = 0x44524F50u;
+    uint32_t k0 = (uint32_t)(seed & 0xffffffffull), k1 = (uint32_t)(seed >> 32);
+    for (int round = 0; round < 10; ++round) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    const uint32_t w[4] = {c0, c1, c2, c3};
+    const int r = 4 * ((j & 31) >> 3) + (j & 3);
+    return (int)((w[r >> 2] >> (8 * (r & 3))) & 255u) >= threshold;
+}
+
 int fa_fwd_validate(const fa_fwd_params *p)
 {
     if (!p || !p->Q || !p->K || !p->V || !p->O) return FA_ERR_NULL_POINTER;
     if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
     if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
     if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
-    if (p->dropout_prob != 0.0f || p->states != nullptr) return FA_ERR_UNSUPPORTED;
+    if (!(p->dropout_prob >= 0.0f) || !(p->dropout_prob < 1.0f)) return FA_ERR_UNSUPPORTED;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
@@ -252,7 +277,12 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         }
     }
     const int shape = waves == 8 ? 0 : 1;
-    hipError_t e = (general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
+    // dropout: p in units of 1/256 (a key is kept iff its random byte is >= the threshold)
+    a.drop_threshold = (unsigned)fa_dropout_threshold(p->dropout_prob);
+    a.drop_scale = 256.0f / (256.0f - (float)a.drop_threshold);
+    a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
+    a.seed_hi = (unsigned)(p->seed >> 32);
+    hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
     return FA_OK;
@@ -264,7 +294,6 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
 {
     (void)M;
     (void)states;
-    if (Is_dropout) return FA_ERR_UNSUPPORTED;
     if (Has_alibi && alibi_slopes == nullptr) return FA_ERR_NULL_POINTER;
     if (d <= 0) return FA_ERR_HEAD_DIM;
     fa_fwd_params p;
@@ -273,7 +302,8 @@ int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, v
     p.L = static_cast<float *>(L);
     p.B = B; p.N = N; p.S = S; p.d = d;
     p.softmax_scale = (float)(1.0 / sqrt((double)d));      // flash_forward.h:639
-    p.dropout_prob = dropout_prob;
+    p.dropout_prob = Is_dropout ? dropout_prob : 0.0f;
+    p.seed = 48;                                             // the seed main() gives its curand states, main.cu:93
     p.alibi_slopes_ptr = Has_alibi ? alibi_slopes : nullptr;      // [N] device floats, main.cu:36-45
     p.window_size_left = Is_local ? window_size : -1;      // flash_forward.h:640-641, mask.h:55
     p.window_size_right = Is_local ? window_size : -1;

@@ -17,5 +17,5 @@ int fa_work_queue_slots() { return kQueueSlots; }
 hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                         hipStream_t stream)
 {
-    return launch_forward<false>(a, bf16, D, masked, shape, grid, stream);
+    return launch_forward<false, false>(a, bf16, D, masked, shape, grid, stream);
 }

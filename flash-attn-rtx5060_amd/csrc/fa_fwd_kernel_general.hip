@@ -5,5 +5,5 @@
 hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream)
 {
-    return launch_forward<true>(a, bf16, D, masked, shape, grid, stream);
+    return launch_forward<true, false>(a, bf16, D, masked, shape, grid, stream);
 }

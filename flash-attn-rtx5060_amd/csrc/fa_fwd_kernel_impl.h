@@ -144,6 +144,34 @@ template <int V> struct IntC { static constexpr int value = V; };
 // ---------------------------------------------------------------------------
 constexpr int kFaithfulRows = 32;
 
+// ---------------------------------------------------------------------------
+// Dropout (role of reference src/flash_forward.h:248-265: after the softmax every P element is zeroed with
+// probability p or multiplied by 1/(1-p); the row sums keep the undropped values).  The reference draws from
+// per-thread curand states, which nothing can replay; here the decision is a pure function of
+// (seed, batch*heads + head, query i, key j): one Philox4x32-10 block yields sixteen bytes for the sixteen keys
+// j of a 32-key block that have the same (j / 4) % 2 -- exactly the keys of that block one lane of this kernel
+// holds for its query -- and key j is kept iff its byte is >= the threshold (p in units of 1/256).
+//   counter = (2 * (j / 32) + (j / 4) % 2,  i,  batch*heads + head,  0x44524F50),  key = (seed lo, seed hi)
+//   byte index = 4 * ((j % 32) / 8) + j % 4, bytes numbered from the low byte of output word 0
+// ---------------------------------------------------------------------------
+struct DropWords { uint32_t w[4]; };
+__device__ __forceinline__ DropWords dropout_words(uint32_t seed_lo, uint32_t seed_hi, uint32_t bh, uint32_t i, uint32_t group)
+{
+    uint32_t c0 = group, c1 = i, c2 = bh, c3 = 0x44524F50u, k0 = seed_lo, k1 = seed_hi;
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const uint32_t h0 = __umulhi(0xD2511F53u, c0), l0 = 0xD2511F53u * c0;
+        const uint32_t h1 = __umulhi(0xCD9E8D57u, c2), l1 = 0xCD9E8D57u * c2;
+        c0 = h1 ^ c1 ^ k0; c1 = l1; c2 = h0 ^ c3 ^ k1; c3 = l0;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    return DropWords{{c0, c1, c2, c3}};
+}
+__device__ __forceinline__ bool dropout_keep_byte(const DropWords &d, int r, uint32_t threshold)
+{
+    return ((d.w[r >> 2] >> (8 * (r & 3))) & 255u) >= threshold;
+}
+
 template <bool BF16> __device__ __forceinline__ float storage_to_f32(uint16_t h)
 {
     if (BF16) return __builtin_bit_cast(float, (uint32_t)h << 16);
@@ -164,6 +192,7 @@ template <bool BF16, int D>
 __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
                                     float *lse_h, int S, int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
+                                    uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
                                     float *sc /* LDS, 32*32 floats */)
 {
     constexpr int R = kFaithfulRows;
@@ -191,7 +220,14 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
         for (int j = 0; j <= tid; ++j) mx = fmaxf(mx, row[j]);
         float sum = 0.0f;
         for (int j = 0; j <= tid; ++j) { row[j] = expf(row[j] - mx); sum += row[j]; }
-        for (int j = 0; j <= tid; ++j) row[j] = storage_to_f32<BF16>(f32_to_storage<BF16>(row[j] / sum));
+        for (int j = 0; j <= tid; ++j) {
+            float pj = row[j] / sum;
+            if (drop_threshold != 0u) {        // keys 0..31: one 32-key block, two Philox blocks per query
+                const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)tid, (uint32_t)((j >> 2) & 1));
+                pj = dropout_keep_byte(d, 4 * (j >> 3) + (j & 3), drop_threshold) ? __fmul_rn(pj, drop_scale) : 0.0f;
+            }
+            row[j] = storage_to_f32<BF16>(f32_to_storage<BF16>(pj));
+        }
         if (lse_h != nullptr) lse_h[tid] = mx + logf(sum);
     }
     __syncthreads();
@@ -216,7 +252,7 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST>
 __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
 {
     constexpr int WR = 32 * RB;                   // query rows per wave
@@ -506,7 +542,23 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // dropout decisions of the tile whose exponentials come next: per row block and key block the sixteen
+    // bytes for this lane's sixteen keys
+    DropWords dw[RB][2];
+    auto draw_dropout = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)bh, (uint32_t)(my_q + 32 * b),
+                                          (uint32_t)(2 * (2 * tile + kb) + half));
+    };
+    auto dropped = [&](float e, int b, int kb, int r) __attribute__((always_inline)) {
+        if (!DROPOUT) return e;
+        return dropout_keep_byte(dw[b][kb], r, a.drop_threshold) ? e * a.drop_scale : 0.0f;
+    };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
+        if (DROPOUT) draw_dropout(tile);
         if (ALIBI) apply_alibi(tile);
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
 #pragma unroll
@@ -522,8 +574,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                 const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], cs, -mc));
                 const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], cs, -mc));
                 l_a[b] += e0; l_b[b] += e1; l_a[b] += e2; l_b[b] += e3;
-                pk[b][i] = N::pack2(e0, e1);
-                pk[b][8 + i] = N::pack2(e2, e3);
+                pk[b][i] = N::pack2(dropped(e0, b, 0, 2 * i), dropped(e1, b, 0, 2 * i + 1));
+                pk[b][8 + i] = N::pack2(dropped(e2, b, 1, 2 * i), dropped(e3, b, 1, 2 * i + 1));
             }
         }
     };
@@ -539,6 +591,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         };
 #pragma unroll
         for (int n = 0; n < PD; ++n) fetch(n);
+        if (DROPOUT) draw_dropout(tile);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
         if (ALIBI) apply_alibi(tile);
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
@@ -584,7 +637,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     const float e1 = __builtin_amdgcn_exp2f(ALIBI ? x1 + nmc[pb] : __builtin_fmaf(x1, c, nmc[pb]));
                     l_a[pb] += e0;
                     l_b[pb] += e1;
-                    uint32_t packed = N::pack2(e0, e1);
+                    uint32_t packed = N::pack2(dropped(e0, pb, e >> 3, 2 * (e & 7)), dropped(e1, pb, e >> 3, 2 * (e & 7) + 1));
                     asm volatile("" : "+v"(packed), "+v"(l_a[pb]), "+v"(l_b[pb]));
                     pn[pb][e] = packed;
                 }
@@ -690,7 +743,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     }
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
-                                     slope, q_rs, k_rs, v_rs, o_rs, reinterpret_cast<float *>(smem));
+                                     slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale, a.seed_lo,
+                                     a.seed_hi, (uint32_t)bh, reinterpret_cast<float *>(smem));
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
     if (a.queue != nullptr && tid == 0) {
@@ -702,12 +756,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     }
 }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST>
 hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
     const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, NW, RB, NST>;
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
@@ -719,14 +773,14 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 // shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
 // (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
 // answers it with about 500 AGPR<->VGPR moves per tile.)
-template <bool GENERAL>
+template <bool GENERAL, bool DROPOUT>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, 8, 1, 3>(a, grid, stream); \
-        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, 4, 1, 2>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, 3>(a, grid, stream); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
     FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)

@@ -29,6 +29,10 @@ struct FaKernelArgs {
     int q_rs, k_rs, v_rs, o_rs;                 // row (sequence position) strides
     long long q_bs, q_hs, k_bs, k_hs;           // batch and head strides
     long long v_bs, v_hs, o_bs, o_hs;
+    // --- used by the DROPOUT instantiations only
+    unsigned drop_threshold;   // key kept iff its byte >= threshold; p = threshold / 256
+    float drop_scale;          // 256 / (256 - threshold)
+    unsigned seed_lo, seed_hi;
 };
 
 #endif

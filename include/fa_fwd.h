@@ -30,7 +30,7 @@ enum {
     FA_ERR_HEAD_DIM = -3,          /* d not in {64, 128}: reference throws, flash_forward.h:587 */
     FA_ERR_SEQLEN_MULTIPLE = -4,   /* reserved (was: S % 128 != 0, which the reference assumes silently,
                                       :134,637); any S >= 1 is accepted now                 */
-    FA_ERR_UNSUPPORTED = -5,       /* dropout requested                                      */
+    FA_ERR_UNSUPPORTED = -5,       /* dropout_prob is not in [0, 1)                          */
     FA_ERR_DTYPE = -6,             /* dtype is neither FA_DTYPE_F16 nor FA_DTYPE_BF16        */
     FA_ERR_SCALE = -7,             /* softmax_scale is not a finite positive number          */
     FA_ERR_DEVICE = -8,            /* a HIP runtime call failed; see fa_last_device_error()  */
@@ -74,9 +74,10 @@ typedef struct fa_fwd_params {
     int Tr;                   /* ignored on input (the reference derives them, :637-638)      */
     int Tc;
     float softmax_scale;      /* the reference sets 1/sqrt(d) itself, flash_forward.h:639     */
-    float dropout_prob;       /* must be 0                                                    */
-    unsigned long long seed;  /* unused                                                       */
-    void *states;             /* dropout RNG states: must be NULL                             */
+    float dropout_prob;       /* in [0, 1), applied in units of 1/256 (fa_dropout_threshold); 0 = none */
+    unsigned long long seed;  /* dropout seed: the kept keys are a function of (seed, batch*N + head,
+                                 query, key) alone, see fa_dropout_keep                       */
+    void *states;             /* the reference's curand states (flash_forward.h:611): ignored */
     int window_size_left;     /* keys with i - j > left are masked;  < 0 = unbounded          */
     int window_size_right;    /* keys with j - i > right are masked; < 0 = unbounded          */
     const float *alibi_slopes_ptr; /* [N] device floats: score -= slope[h]*|i-j| (mask.h:21-26), or NULL */
@@ -116,7 +117,9 @@ int fa_fwd(const fa_fwd_params *p, void *stream);
  * prints nothing, returns a status, and fills L with the fp32 logsumexp when
  * L is non-NULL.  M is ignored.  `Has_alibi` takes `alibi_slopes` as N device floats and subtracts
  * slope[h]*|i-j| from every scaled score, once (mask.h:21-26; the reference applies it twice when causal
- * and local are both set).  Dropout returns FA_ERR_UNSUPPORTED.
+ * and local are both set).  `Is_dropout` applies dropout_prob with the fixed seed 48 (the seed main() gives its
+ * curand states, main.cu:93); `states` is ignored: the kept keys come from a counter-based generator that a
+ * host can replay (fa_dropout_keep), which curand states do not allow.
  */
 int run_flash_attention(int B, int N, int S, int d,
                         void *Q, void *K, void *V, void *O,
@@ -124,6 +127,17 @@ int run_flash_attention(int B, int N, int S, int d,
                         int Is_dropout, int Is_causal, int Is_local, int Has_alibi,
                         int window_size, float *alibi_slopes,
                         float dropout_prob, void *states);
+
+/*
+ * Dropout (reference flash_forward.h:248-265: after the softmax each probability is zeroed with probability p
+ * or multiplied by 1/(1-p); the logsumexp is that of the undropped scores).  The decision for (bh = batch*N +
+ * head, query i, key j) is byte 4*((j%32)/8) + j%4 of the Philox4x32-10 block with counter
+ * (2*(j/32) + (j/4)%2, i, bh, 0x44524F50) and key (seed low, seed high): the key is kept iff that byte is >=
+ * the threshold.  fa_dropout_threshold(p) = p rounded to 1/256 (at most 255); the factor applied to kept keys
+ * is 256 / (256 - threshold).  Both are host functions: a backward pass or a test can replay the mask.
+ */
+int fa_dropout_threshold(float dropout_prob);
+int fa_dropout_keep(unsigned long long seed, long long bh, int i, int j, int threshold);
 
 const char *fa_strerror(int status);
 /* Text of the last HIP error seen by the calling thread ("" if none). */

@@ -118,7 +118,41 @@ static inline int masked(const fa_oracle_cfg *c, int i, int j)
 static int cfg_ok(const fa_oracle_cfg *c)
 {
     return c && c->B > 0 && c->H > 0 && c->S > 0 && c->D > 0 &&
-           (c->dtype == FA_ORACLE_F16 || c->dtype == FA_ORACLE_BF16);
+           (c->dtype == FA_ORACLE_F16 || c->dtype == FA_ORACLE_BF16) &&
+           c->dropout_threshold >= 0 && c->dropout_threshold <= 255;
+}
+
+/* ------------------------------------------------------------------ */
+/* dropout: a counter-based decision per (head, query, key)            */
+/* ------------------------------------------------------------------ */
+void fa_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c[4] = {ctr[0], ctr[1], ctr[2], ctr[3]}, k[2] = {key[0], key[1]};
+    for (int round = 0; round < 10; ++round) {
+        const uint64_t lo = (uint64_t)0xD2511F53u * c[0], hi = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n[4] = {(uint32_t)(hi >> 32) ^ c[1] ^ k[0], (uint32_t)hi, (uint32_t)(lo >> 32) ^ c[3] ^ k[1], (uint32_t)lo};
+        memcpy(c, n, sizeof(c));
+        k[0] += 0x9E3779B9u;        /* golden-ratio and sqrt(3)-1 Weyl increments */
+        k[1] += 0xBB67AE85u;
+    }
+    memcpy(out, c, sizeof(c));
+}
+
+int fa_oracle_dropout_keep(uint64_t seed, int64_t bh, int i, int j, int threshold)
+{
+    const uint32_t ctr[4] = {(uint32_t)(2 * (j / 32) + (j / 4) % 2), (uint32_t)i, (uint32_t)bh, 0x44524F50u};
+    const uint32_t key[2] = {(uint32_t)(seed & 0xffffffffu), (uint32_t)(seed >> 32)};
+    uint32_t w[4];
+    fa_oracle_philox4x32_10(ctr, key, w);
+    const int byte = 4 * ((j % 32) / 8) + j % 4;
+    return (int)((w[byte / 4] >> (8 * (byte % 4))) & 255u) >= threshold;
+}
+/* p after dropout (fp32: one rounding for the division that produced p, one for the product) */
+static inline float drop_f32(const fa_oracle_cfg *c, int64_t bh, int i, int j, float p)
+{
+    if (c->dropout_threshold == 0) return p;
+    if (!fa_oracle_dropout_keep(c->dropout_seed, bh, i, j, c->dropout_threshold)) return 0.0f;
+    return p * (256.0f / (256.0f - (float)c->dropout_threshold));
 }
 
 /* ------------------------------------------------------------------ */
@@ -160,7 +194,7 @@ int fa_oracle_literal(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t 
                 for (int j = 0; j < S; ++j) mx = fmaxf(mx, row[j]);
                 float sum = 0.0f;
                 for (int j = 0; j < S; ++j) { row[j] = expf(row[j] - mx); sum += row[j]; }
-                for (int j = 0; j < S; ++j) row[j] /= sum;
+                for (int j = 0; j < S; ++j) row[j] = drop_f32(c, (int64_t)b * c->H + h, i, j, row[j] / sum);
             }
             for (int i = 0; i < S; ++i)
                 for (int t = 0; t < D; ++t) {
@@ -311,7 +345,7 @@ int fa_oracle_rows(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t *K,
             for (int j = lo; j <= hi; ++j) mx = fmaxf(mx, sc[j - lo]);
             float sum = 0.0f;
             for (int j = lo; j <= hi; ++j) { sc[j - lo] = expf(sc[j - lo] - mx); sum += sc[j - lo]; }
-            for (int j = lo; j <= hi; ++j) sc[j - lo] = widen(narrow(sc[j - lo] / sum, dt), dt);
+            for (int j = lo; j <= hi; ++j) sc[j - lo] = widen(narrow(drop_f32(c, bh, i, j, sc[j - lo] / sum), dt), dt);
             if (O_rows) {
                 row_pv(c, sc, Vf, lo, hi, out);
                 for (int t = 0; t < D; ++t) O_rows[(size_t)order[n].pos * D + t] = narrow(out[t], dt);
@@ -371,7 +405,10 @@ int fa_oracle_rows_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t
         if (O_rows) {
             for (int t = 0; t < D; ++t) out[t] = 0.0;
             for (int j = lo; j <= hi; ++j) {
-                const double p = sc[j - lo] / sum;
+                double p = sc[j - lo] / sum;
+                if (c->dropout_threshold != 0)
+                    p = fa_oracle_dropout_keep(c->dropout_seed, bh, i, j, c->dropout_threshold)
+                            ? p * (256.0 / (256.0 - (double)c->dropout_threshold)) : 0.0;
                 for (int t = 0; t < D; ++t) out[t] += p * (double)widen(v[(size_t)j * D + t], dt);
             }
             for (int t = 0; t < D; ++t) O_rows[(size_t)n * D + t] = out[t];

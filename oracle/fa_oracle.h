@@ -36,7 +36,20 @@ typedef struct fa_oracle_cfg {
                            /* reference window_size w (main.cu:220-229) is
                               window_left = window_right = w                  */
     const float *alibi_slopes; /* [H] or NULL, main.cu:200-207                */
+    /* Dropout (GPU side of the reference only, flash_forward.h:248-265; its CPU verifier skips dropout runs,
+       main.cu:102): every normalised probability is zeroed when its random byte is below the threshold and
+       multiplied by 256/(256-threshold) otherwise, before it is rounded to the storage type; the logsumexp is
+       untouched.  threshold 0 = no dropout. */
+    int dropout_threshold;     /* 0..255: drop probability in units of 1/256  */
+    uint64_t dropout_seed;
 } fa_oracle_cfg;
+
+/* The dropout decision for (bh = b*H + h, query i, key j): 1 = kept.  Byte 4*((j%32)/8) + j%4 of the
+ * Philox4x32-10 block with counter (2*(j/32) + (j/4)%2, i, bh, 0x44524F50) and key (seed low, seed high),
+ * compared with the threshold. */
+int fa_oracle_dropout_keep(uint64_t seed, int64_t bh, int i, int j, int threshold);
+/* Philox4x32-10 as published (Salmon et al., Random123), exposed for its known-answer tests. */
+void fa_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
 
 /* Scalar conversions (round-to-nearest-even), exposed for the tests. */
 uint16_t fa_oracle_f32_to_f16(float x);

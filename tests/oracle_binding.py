@@ -11,7 +11,8 @@ F16, BF16 = 0, 1
 class Cfg(ctypes.Structure):
     _fields_ = [("B", ctypes.c_int), ("H", ctypes.c_int), ("S", ctypes.c_int), ("D", ctypes.c_int),
                 ("dtype", ctypes.c_int), ("scale", ctypes.c_float), ("causal", ctypes.c_int),
-                ("window_left", ctypes.c_int), ("window_right", ctypes.c_int), ("alibi_slopes", ctypes.c_void_p)]
+                ("window_left", ctypes.c_int), ("window_right", ctypes.c_int), ("alibi_slopes", ctypes.c_void_p),
+                ("dropout_threshold", ctypes.c_int), ("dropout_seed", ctypes.c_uint64)]
 
 
 _libs = {}
@@ -37,13 +38,16 @@ def lib(scalar=False):
         L.fa_oracle_full.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp, vp, ctypes.c_int]
         L.fa_oracle_rows_f64.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp, ctypes.c_int64, vp, vp, ctypes.c_int]
         L.fa_oracle_literal.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp]
+        L.fa_oracle_dropout_keep.argtypes = [ctypes.c_uint64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        L.fa_oracle_philox4x32_10.restype = None
+        L.fa_oracle_philox4x32_10.argtypes = [ctypes.POINTER(ctypes.c_uint32)] * 3
         _libs[name] = L
     return _libs[name]
 
 
-def _cfg(shape, dtype, scale, causal, wl, wr, slopes):
+def _cfg(shape, dtype, scale, causal, wl, wr, slopes, dropout=(0, 0)):
     B, H, S, D = shape
-    c = Cfg(B, H, S, D, dtype, scale, int(bool(causal)), wl, wr, None)
+    c = Cfg(B, H, S, D, dtype, scale, int(bool(causal)), wl, wr, None, int(dropout[0]), int(dropout[1]))
     if slopes is not None:
         c.alibi_slopes = slopes.ctypes.data
     return c
@@ -58,47 +62,49 @@ def default_threads():
     return max(1, min(16, os.cpu_count() or 1))
 
 
-def rows(q, k, v, row_idx, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, scalar=False):
-    """Faithful oracle on selected flat rows -> (O [n, D] uint16 bits, lse [n] float32)."""
+def rows(q, k, v, row_idx, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, scalar=False,
+         dropout=(0, 0)):
+    """Faithful oracle on selected flat rows -> (O [n, D] uint16 bits, lse [n] float32).
+    dropout = (threshold 0..255, seed)."""
     _check((q, k, v))
     B, H, S, D = q.shape
     scale = np.float32(1.0 / np.sqrt(D)) if scale is None else np.float32(scale)
     idx = np.ascontiguousarray(row_idx, dtype=np.int64)
     o = np.empty((len(idx), D), dtype=np.uint16)
     lse = np.empty((len(idx),), dtype=np.float32)
-    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes)
+    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes, dropout)
     rc = lib(scalar).fa_oracle_rows(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, idx.ctypes.data,
                                     len(idx), o.ctypes.data, lse.ctypes.data, threads or default_threads())
     assert rc == 0
     return o, lse
 
 
-def full(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, scalar=False):
+def full(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, scalar=False, dropout=(0, 0)):
     B, H, S, D = q.shape
-    o, lse = rows(q, k, v, np.arange(B * H * S, dtype=np.int64), dtype, scale, causal, wl, wr, slopes, threads, scalar)
+    o, lse = rows(q, k, v, np.arange(B * H * S, dtype=np.int64), dtype, scale, causal, wl, wr, slopes, threads, scalar, dropout)
     return o.reshape(B, H, S, D), lse.reshape(B, H, S)
 
 
-def rows_f64(q, k, v, row_idx, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None):
+def rows_f64(q, k, v, row_idx, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, dropout=(0, 0)):
     _check((q, k, v))
     B, H, S, D = q.shape
     scale = np.float32(1.0 / np.sqrt(D)) if scale is None else np.float32(scale)
     idx = np.ascontiguousarray(row_idx, dtype=np.int64)
     o = np.empty((len(idx), D), dtype=np.float64)
     lse = np.empty((len(idx),), dtype=np.float64)
-    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes)
+    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes, dropout)
     rc = lib().fa_oracle_rows_f64(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, idx.ctypes.data,
                                   len(idx), o.ctypes.data, lse.ctypes.data, threads or default_threads())
     assert rc == 0
     return o, lse
 
 
-def literal(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, scalar=False):
+def literal(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, scalar=False, dropout=(0, 0)):
     _check((q, k, v))
     B, H, S, D = q.shape
     scale = np.float32(1.0 / np.sqrt(D)) if scale is None else np.float32(scale)
     o = np.empty((B, H, S, D), dtype=np.uint16)
-    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes)
+    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes, dropout)
     rc = lib(scalar).fa_oracle_literal(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data)
     assert rc == 0
     return o

@@ -62,3 +62,26 @@ def sample_rows(shape, n, seed, extra=()):
     if want:
         rows.extend(rng.integers(0, B * H * S, size=want).tolist())
     return np.unique(np.asarray(rows, dtype=np.int64))
+
+
+def numpy_philox4x32_10(ctr, key):
+    """Philox4x32-10 on numpy uint64 arrays of counters (an implementation independent of the C ones)."""
+    c = [np.asarray(x, dtype=np.uint64) for x in ctr]
+    k = [np.uint64(key[0]), np.uint64(key[1])]
+    m32 = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0 = np.uint64(0xD2511F53) * c[0]
+        p1 = np.uint64(0xCD9E8D57) * c[2]
+        c = [(p1 >> np.uint64(32)) ^ c[1] ^ k[0], p1 & m32, (p0 >> np.uint64(32)) ^ c[3] ^ k[1], p0 & m32]
+        k = [(k[0] + np.uint64(0x9E3779B9)) & m32, (k[1] + np.uint64(0xBB67AE85)) & m32]
+    return c
+
+
+def numpy_keep_mask(seed, bh, S, threshold):
+    """keep[i, j] from the published definition of the dropout decision, vectorised over (i, j)."""
+    i, j = np.meshgrid(np.arange(S), np.arange(S), indexing="ij")
+    w = numpy_philox4x32_10((2 * (j // 32) + (j // 4) % 2, i, np.full_like(i, bh), np.full_like(i, 0x44524F50)),
+                            (seed & 0xFFFFFFFF, seed >> 32))
+    byte = 4 * ((j % 32) // 8) + j % 4
+    word = np.choose(byte // 4, w)
+    return ((word >> (8 * (byte % 4)).astype(np.uint64)) & np.uint64(255)) >= np.uint64(threshold)

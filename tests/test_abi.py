@@ -3,6 +3,8 @@ rejects bad arguments with status codes (the reference exits/aborts/throws: util
 flash_forward.h:384-387,587-589)."""
 import ctypes
 import os
+
+import numpy as np
 import re
 
 import pytest
@@ -82,8 +84,10 @@ def test_validate_status_codes(fa):
     assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE
     assert status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE
     assert status(softmax_scale=float("inf")) == fa.FA_ERR_SCALE
-    assert status_raw(dict(dropout_prob=0.1)) == fa.FA_ERR_UNSUPPORTED
-    assert status_raw(dict(states=0x10)) == fa.FA_ERR_UNSUPPORTED
+    assert status_raw(dict(dropout_prob=0.1)) == fa.FA_OK                    # dropout is accepted ...
+    assert status_raw(dict(states=0x10)) == fa.FA_OK                         # ... the curand states are ignored
+    for bad_p in (1.0, 1.5, -0.1, float("nan")):
+        assert status_raw(dict(dropout_prob=bad_p)) == fa.FA_ERR_UNSUPPORTED
     assert status_raw(dict(alibi_slopes_ptr=0x10)) == fa.FA_OK               # ALiBi slopes are accepted
     assert status(B=70000, N=70000, S=128) == fa.FA_ERR_TOO_LARGE
     # layouts: K/V heads must divide the query heads, strides are multiples of 8 elements with a row stride of
@@ -105,7 +109,7 @@ def test_validate_status_codes(fa):
 def test_reference_entry_point_rejects_unsupported_flags(fa):
     L = fa.lib()
     args = [2, 8, 2048, 64, 0x1000, 0x2000, 0x3000, 0x4000, None, None]
-    assert L.run_flash_attention(*args, 1, 0, 0, 0, 0, None, 0.0, None) == fa.FA_ERR_UNSUPPORTED   # dropout
+    assert L.run_flash_attention(*args, 1, 0, 0, 0, 0, None, 1.0, None) == fa.FA_ERR_UNSUPPORTED   # dropout with p = 1
     assert L.run_flash_attention(*args, 0, 0, 0, 1, 0, None, 0.0, None) == fa.FA_ERR_NULL_POINTER  # ALiBi without slopes
     bad = list(args)
     bad[3] = 48
@@ -138,3 +142,14 @@ def test_python_wrapper_refuses_cpu_tensors(fa):
     q = torch.zeros(1, 1, 128, 64, dtype=torch.float16)
     with pytest.raises(ValueError):
         fa.flash_attention_forward(q, q, q)
+
+
+def test_dropout_host_mirror(fa):
+    """fa_dropout_threshold rounds p to 1/256; fa_dropout_keep follows the published definition (numpy Philox)."""
+    from parity_util import numpy_keep_mask
+    L = fa.lib()
+    assert [L.fa_dropout_threshold(p) for p in (0.0, -1.0, 0.001, 0.1, 0.5, 0.999, 1.0)] == [0, 0, 0, 26, 128, 255, 255]
+    for seed, bh, thr in ((48, 3, 26), (0xFEDCBA9876543210, 70, 200)):
+        want = numpy_keep_mask(seed, bh, 80, thr)
+        got = np.array([[L.fa_dropout_keep(seed, bh, i, j, thr) for j in range(80)] for i in range(80)], dtype=bool)
+        assert np.array_equal(got, want)

@@ -5,12 +5,14 @@ reference's loop structure vs the streamed evaluation (bit-exact), the bit-level
 closed forms and invariants chosen so that a dropped scale, a wrong mask edge, a transposed operand or a
 missing rounding step fails at least one of them, brute-force fp64 fixtures under tests/golden, and torch's
 scaled_dot_product_attention."""
+import ctypes
 import os
 
 import numpy as np
 import pytest
 
 import oracle_binding as ob
+from parity_util import numpy_keep_mask, numpy_philox4x32_10
 
 F16, BF16 = ob.F16, ob.BF16
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -349,6 +351,66 @@ def test_alibi_against_numpy_f64_and_torch_sdpa(dtype, causal, wl, wr):
     o, lse = ob.full(q, k, v, dtype, None, causal, wl, wr, slopes)
     assert np.max(np.abs(ob.to_f32(o, dtype) - o_np)) <= (3e-3 if dtype == F16 else 1.6e-2)
     assert np.max(np.abs(lse - lse_np)) <= (2e-3 if dtype == F16 else 8e-3)
+
+
+# ---------------------------------------------------------------- dropout (flash_forward.h:248-265)
+def test_dropout_philox_known_answers_and_mask_definition():
+    L = ob.lib()
+
+    def philox(ctr, key):
+        c, k, o = (ctypes.c_uint32 * 4)(*ctr), (ctypes.c_uint32 * 2)(*key), (ctypes.c_uint32 * 4)()
+        L.fa_oracle_philox4x32_10(c, k, o)
+        return tuple(o)
+    # Random123 known answers for Philox4x32-10
+    f = 0xFFFFFFFF
+    assert philox((0, 0, 0, 0), (0, 0)) == (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)
+    assert philox((f, f, f, f), (f, f)) == (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)
+    assert philox((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0)) == \
+        (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)
+    assert tuple(int(x) for x in numpy_philox4x32_10((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0))) == \
+        (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)
+    # the C decision function against the numpy one, all (i, j) of a 96 x 96 block, two heads, two thresholds
+    for seed, bh, thr in ((48, 0, 26), (0x1234567890ABCDEF, 5, 128)):
+        want = numpy_keep_mask(seed, bh, 96, thr)
+        got = np.array([[L.fa_oracle_dropout_keep(seed, bh, i, j, thr) for j in range(96)] for i in range(96)], dtype=bool)
+        assert np.array_equal(got, want)
+        assert abs(want.mean() - (1 - thr / 256)) < 4 * np.sqrt(thr / 256 * (1 - thr / 256) / want.size)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_dropout_mask_read_back_through_identity_values(causal):
+    """Q = 0 makes P uniform over the n_i visible keys; V = identity then gives O_ij = keep_ij / (n_i (1-p)):
+    the mask the oracle applied is read off its output and compared with the numpy definition, and the
+    logsumexp must be that of the run without dropout."""
+    H, S, thr, seed = 2, 64, 77, 0xC0FFEE
+    q = np.zeros((1, H, S, S), dtype=np.uint16)
+    k = rand_bits(np.random.default_rng(3), (1, H, S, S), F16)
+    v = np.broadcast_to(ob.from_f32(np.eye(S, dtype=np.float32), F16), (1, H, S, S)).copy()
+    o64, lse64 = ob.rows_f64(q, k, v, np.arange(H * S), F16, None, causal, -1, -1, None, dropout=(thr, seed))
+    o, lse = ob.full(q, k, v, F16, None, causal, -1, -1, None, dropout=(thr, seed))
+    _, lse_plain = ob.full(q, k, v, F16, None, causal, -1, -1)
+    assert np.array_equal(lse, lse_plain)
+    i, j = np.meshgrid(np.arange(S), np.arange(S), indexing="ij")
+    vis = (j <= i) if causal else np.ones((S, S), dtype=bool)
+    n = vis.sum(axis=1, keepdims=True)
+    for h in range(H):
+        want = np.where(vis & numpy_keep_mask(seed, h, S, thr), 1.0 / (n * (1 - thr / 256)), 0.0)
+        assert np.allclose(o64.reshape(H, S, S)[h], want, atol=1e-12)
+        assert np.max(np.abs(ob.to_f32(o, F16)[0, h] - want)) <= 1e-3 * np.maximum(want.max(), 1.0)
+
+
+def test_dropout_threshold_zero_is_no_dropout_and_streamed_equals_literal():
+    rng = np.random.default_rng(21)
+    shape = (1, 2, 72, 32)
+    q, k, v = (rand_bits(rng, shape, F16) for _ in range(3))
+    o0, l0 = ob.full(q, k, v, F16, None, True, -1, -1)
+    o1, l1 = ob.full(q, k, v, F16, None, True, -1, -1, None, dropout=(0, 12345))
+    assert np.array_equal(o0, o1) and np.array_equal(l0, l1)
+    for dtype in (F16, BF16):
+        lit = ob.literal(q, k, v, dtype, None, True, 40, -1, None, dropout=(60, 9))
+        o, _ = ob.full(q, k, v, dtype, None, True, 40, -1, None, dropout=(60, 9))
+        o_s, _ = ob.full(q, k, v, dtype, None, True, 40, -1, None, scalar=True, dropout=(60, 9))
+        assert np.array_equal(o, lit) and np.array_equal(o_s, lit)
 
 
 def test_golden_fixture_f64():
