@@ -15,7 +15,11 @@
  * agreement with the CUDA host `__half` operators of the reference build is
  * "parity unpinned": it follows from source semantics (float multiply of two
  * halves is exact, then one round-to-nearest-even) but no reference binary
- * can be run here.
+ * can be run here.  Dropout is also "parity unpinned" against the reference,
+ * by construction: the reference's kernel draws from per-thread curand states
+ * and its verifier skips dropout runs (main.cu:102); the decision function
+ * used here is a counter-based replacement, pinned by the Random123 known
+ * answers, a numpy implementation and a mask read-back in the same tests.
  */
 #ifndef FA_ORACLE_H
 #define FA_ORACLE_H
