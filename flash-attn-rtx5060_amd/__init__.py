@@ -36,6 +36,7 @@ FA_ERR_DEVICE = -8
 FA_ERR_NO_DEVICE = -9
 FA_ERR_TOO_LARGE = -10
 FA_ERR_LAYOUT = -11
+FA_ERR_WORKSPACE = -12
 FA_DTYPE_F16 = 0
 FA_DTYPE_BF16 = 1
 FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT, FA_SCHED_QUEUE = 0, 1, 2, 3
@@ -46,7 +47,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_validate", "fa_fwd", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
-    "fa_dropout_threshold", "fa_dropout_keep",
+    "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
     "fa_event_elapsed_ms", "fa_event_destroy",
@@ -68,6 +69,7 @@ class FaFwdParams(ctypes.Structure):
         ("n_kv_heads", ctypes.c_int),
         ("q_strides", ctypes.c_longlong * 3), ("k_strides", ctypes.c_longlong * 3),
         ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
+        ("S_kv", ctypes.c_int), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_ulonglong),
     ]
 
 
@@ -101,6 +103,9 @@ def lib():
         L.fa_last_device_error.restype = ctypes.c_char_p
         L.fa_fwd_validate.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.fa_fwd.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
+        L.fa_fwd_workspace_bytes.restype = ctypes.c_ulonglong
+        L.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaFwdParams)]
+        L.fa_fwd_suggest_splits.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.run_flash_attention.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
         L.fa_sched_block_rows.argtypes = [ctypes.c_int] * 4
@@ -148,12 +153,14 @@ def host_lib():
 
 def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
                 window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0,
-                n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None, dropout_prob=0.0, seed=0):
+                n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None, dropout_prob=0.0, seed=0,
+                S_kv=0, split_num=0, workspace_ptr=0, workspace_bytes=0):
     """A filled fa_fwd_params.  Strides are (batch, head, row) in elements, None = contiguous [B,N,S,d]."""
     p = FaFwdParams()
     p.alibi_slopes_ptr = alibi_ptr or None
     p.n_kv_heads = n_kv_heads
     p.dropout_prob, p.seed = dropout_prob, seed
+    p.S_kv, p.split_num, p.workspace, p.workspace_bytes = S_kv, split_num, workspace_ptr or None, workspace_bytes
     for name, st in (("q_strides", q_strides), ("k_strides", k_strides), ("v_strides", v_strides), ("o_strides", o_strides)):
         if st is not None:
             setattr(p, name, (ctypes.c_longlong * 3)(*st))
@@ -167,23 +174,26 @@ def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softm
 
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
                             return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None,
-                            dropout_prob=0.0, seed=0):
+                            dropout_prob=0.0, seed=0, splits=1):
     """O, LSE = attention(q, k, v) on the GPU through fa_fwd().  q is [B, N, S, d], k and v are
     [B, Nk, S, d] with Nk dividing N (Nk < N: grouped-query attention); any strides with a contiguous last
     dimension are passed through (a [B, S, N, d] tensor is given as ``t.transpose(1, 2)``), any S >= 1.
+    k and v may be longer or shorter than q ([B, Nk, S_kv, d]): query i then sits at key position
+    i + S_kv - S.  ``splits``: an int > 1, or "auto", splits the keys of every query block over several
+    workgroups and merges the partial results (few queries, long keys).
     ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26)."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise ValueError("q, k, v must live on the GPU")
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise ValueError("q, k, v must share dtype float16 or bfloat16")
-    if q.dim() != 4 or k.shape != v.shape or k.dim() != 4 or (q.shape[0], q.shape[2], q.shape[3]) != (
-            k.shape[0], k.shape[2], k.shape[3]) or k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0:
-        raise ValueError("q must be [B, N, S, d], k and v [B, Nk, S, d] with Nk dividing N")
+    if q.dim() != 4 or k.shape != v.shape or k.dim() != 4 or (q.shape[0], q.shape[3]) != (
+            k.shape[0], k.shape[3]) or k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0 or k.shape[2] == 0:
+        raise ValueError("q must be [B, N, S, d], k and v [B, Nk, S_kv, d] with Nk dividing N")
     if q.stride(3) != 1 or k.stride(3) != 1 or v.stride(3) != 1:
         raise ValueError("the head dimension of q, k, v must be contiguous")
     B, N, S, d = q.shape
-    Nk = k.shape[1]
+    Nk, S_kv = k.shape[1], k.shape[2]
     if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
                                          and alibi_slopes.is_contiguous() and tuple(alibi_slopes.shape) == (N,)):
         raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
@@ -198,7 +208,16 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
                     FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched,
                     0 if alibi_slopes is None else alibi_slopes.data_ptr(), 0 if Nk == N else Nk,
                     *[None if t.is_contiguous() else tuple(t.stride()[:3]) for t in (q, k, v, out)],
-                    dropout_prob=dropout_prob, seed=seed)
+                    dropout_prob=dropout_prob, seed=seed, S_kv=0 if S_kv == S else S_kv)
+    if splits == "auto":
+        splits = lib().fa_fwd_suggest_splits(ctypes.byref(p))
+    workspace = None
+    if splits and splits > 1:
+        p.split_num = int(splits)
+        need = lib().fa_fwd_workspace_bytes(ctypes.byref(p))
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)   # stream-ordered: freed after the launch
+            p.workspace, p.workspace_bytes = workspace.data_ptr(), need
     stream = torch.cuda.current_stream(q.device).cuda_stream
     st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
     if st != FA_OK:

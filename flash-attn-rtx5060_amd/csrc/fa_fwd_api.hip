@@ -23,6 +23,7 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
                                      hipStream_t stream);
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
+hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -82,6 +83,7 @@ const char *fa_strerror(int status)
     case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
     case FA_ERR_SEQLEN_MULTIPLE: return "reserved (seqlen no longer has to be a multiple of 128)";
+    case FA_ERR_WORKSPACE: return "split_num > 1 needs a 16-byte aligned workspace of fa_fwd_workspace_bytes() bytes";
     case FA_ERR_LAYOUT: return "strides must be multiples of 8 elements (row strides at least head_dim), n_kv_heads must divide heads, pointers must be 16-byte aligned";
     case FA_ERR_UNSUPPORTED: return "dropout_prob must be at least 0 and below 1";
     case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
@@ -178,6 +180,39 @@ int fa_dropout_keep(unsigned long long seed, long long bh, int i, int j, int thr
     return (int)((w[r >> 2] >> (8 * (r & 3))) & 255u) >= threshold;
 }
 
+namespace {
+int key_tiles(const fa_fwd_params *p) { return ((p->S_kv > 0 ? p->S_kv : p->S) + kBlockKeysHost - 1) / kBlockKeysHost; }
+// splits actually used: at most one per key tile
+int effective_splits(const fa_fwd_params *p)
+{
+    if (p->split_num <= 1) return 1;
+    const int tiles = key_tiles(p);
+    return p->split_num < tiles ? p->split_num : tiles;
+}
+}  // namespace
+
+unsigned long long fa_fwd_workspace_bytes(const fa_fwd_params *p)
+{
+    if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0 || p->d <= 0) return 0;
+    const int n = effective_splits(p);
+    if (n <= 1) return 0;
+    return (unsigned long long)n * p->B * p->N * p->S * (unsigned long long)(p->d + 1) * 4ull;
+}
+
+int fa_fwd_suggest_splits(const fa_fwd_params *p)
+{
+    if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0) return 1;
+    // work items without splits against the workgroups the device keeps resident; split until the device is
+    // filled about twice, with at least four key tiles (256 keys) per split
+    const long long items = fa_sched_num_items(p->B, p->N, p->S, p->d);
+    const long long resident = (long long)kComputeUnits * (waves_for(p->B, p->N, p->S) == 8 ? 1 : 2);
+    if (items >= resident) return 1;
+    long long n = (2 * resident + items - 1) / items;
+    const long long cap = key_tiles(p) / 4;
+    if (n > cap) n = cap;
+    return n < 1 ? 1 : (int)n;
+}
+
 int fa_fwd_validate(const fa_fwd_params *p)
 {
     if (!p || !p->Q || !p->K || !p->V || !p->O) return FA_ERR_NULL_POINTER;
@@ -188,6 +223,10 @@ int fa_fwd_validate(const fa_fwd_params *p)
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (p->S_kv < 0) return FA_ERR_BAD_SHAPE;
+    if (fa_sched_num_items(p->B, p->N, p->S, p->d) * effective_splits(p) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (effective_splits(p) > 1 && (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
+                                    p->workspace_bytes < fa_fwd_workspace_bytes(p))) return FA_ERR_WORKSPACE;
     if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
     const void *ptrs[4] = {p->Q, p->K, p->V, p->O};
     const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
@@ -220,13 +259,19 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.S = p->S;
     // layout: contiguous [B,N,S,d] unless strides are given; K and V have n_kv_heads heads
     a.Hk = p->n_kv_heads > 0 ? p->n_kv_heads : p->N;
-    bool general = a.Hk != p->N || p->S % 128 != 0;
+    a.Sk = p->S_kv > 0 ? p->S_kv : p->S;
+    a.n_splits = effective_splits(p);
+    a.tiles_per_split = (key_tiles(p) + a.n_splits - 1) / a.n_splits;
+    a.o_part = static_cast<float *>(p->workspace);
+    a.lse_part = a.o_part != nullptr ? a.o_part + (size_t)a.n_splits * p->B * p->N * p->S * p->d : nullptr;
+    bool general = a.Hk != p->N || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
     {
         const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
         long long eff[4][3];
         for (int t = 0; t < 4; ++t) {
             const long long heads = (t == 1 || t == 2) ? a.Hk : p->N;
-            const long long dense[3] = {heads * p->S * p->d, (long long)p->S * p->d, p->d};
+            const long long len = (t == 1 || t == 2) ? a.Sk : p->S;
+            const long long dense[3] = {heads * len * p->d, len * p->d, p->d};
             const long long *st = strides[t];
             const bool given = st[0] != 0 || st[1] != 0 || st[2] != 0;
             for (int k = 0; k < 3; ++k) {
@@ -242,13 +287,14 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     const int waves = waves_for(p->B, p->N, p->S);
     const int block_rows = 32 * waves;
     a.n_qblocks = (p->S + block_rows - 1) / block_rows;
-    fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
+    const int s_max = a.Sk > p->S ? a.Sk : p->S;        // stands in for "unbounded"
+    fa_mask_bounds(s_max, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
     // (a sequence that ends inside a 64-key tile needs the element mask on that tile, whatever the mask)
-    const int masked = (a.L < p->S || a.R < p->S || p->S % kBlockKeysHost != 0) ? 1 : 0;
-    a.descending = (a.L < p->S || a.R < p->S) ? 1 : 0;
+    const int masked = (a.L < s_max || a.R < s_max || a.Sk % kBlockKeysHost != 0) ? 1 : 0;
+    a.descending = (a.L < s_max || a.R < s_max) ? 1 : 0;
     a.scale = p->softmax_scale;
     a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
-    a.n_items = (long long)a.BH * a.n_qblocks;
+    a.n_items = (long long)a.BH * a.n_qblocks * a.n_splits;
 
     // Dispatch mode launches one workgroup per item, in list order; the hardware hands them to CUs as these
     // free up, which is a longest-first greedy schedule.  Persistent mode launches one resident set of
@@ -285,6 +331,10 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
+    if (a.n_splits > 1) {
+        e = fa_launch_combine_splits(a, p->dtype == FA_DTYPE_BF16, p->d, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return device_fail(e, "combine launch");
+    }
     return FA_OK;
 }
 

@@ -53,6 +53,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -190,6 +191,7 @@ template <bool BF16> __device__ __forceinline__ float storage_product(float a, f
 
 template <bool BF16, int D>
 __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
+                                    float *o32 /* null, or [rows][D] fp32 to write instead of Oh */,
                                     float *lse_h, int S, int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
                                     uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
@@ -237,7 +239,8 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
         const int lo = i - L > 0 ? i - L : 0;
         float sum = 0.0f;
         for (int j = lo; j <= i; ++j) sum += storage_product<BF16>(sc[i * R + j], storage_to_f32<BF16>(Vh[(size_t)j * v_rs + t]));
-        Oh[(size_t)i * o_rs + t] = f32_to_storage<BF16>(sum);
+        if (o32 != nullptr) o32[(size_t)i * D + t] = storage_to_f32<BF16>(f32_to_storage<BF16>(sum));
+        else Oh[(size_t)i * o_rs + t] = f32_to_storage<BF16>(sum);
     }
     __syncthreads();
 }
@@ -320,8 +323,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         item = (long long)taken;
     }
     int bh, qblock;
-    fa_item_decode(item, a.BH, a.n_qblocks, a.descending, &bh, &qblock);
+    // (GENERAL with key splits: consecutive list positions are the splits of one (head, query block))
+    const int n_splits = GENERAL ? a.n_splits : 1;
+    const int split = n_splits > 1 ? (int)(item % n_splits) : 0;
+    fa_item_decode(n_splits > 1 ? item / n_splits : item, a.BH, a.n_qblocks, a.descending, &bh, &qblock);
     const int S = a.S;
+    // GENERAL: Sk keys; query i sits at key position i + pos_off (the queries are the last S positions), which
+    // is what masks, the ALiBi distance and the dropout decision see.
+    const int Sk = GENERAL ? a.Sk : S;
+    const int pos_off = GENERAL ? a.Sk - a.S : 0;
     // Contiguous [B,H,S,D] tensors, one K/V head per query head, S a multiple of 128: everything below is
     // compile-time.  GENERAL: any strides (in elements, head dimension contiguous), query heads sharing K/V
     // heads in groups of H/Hk, any S (rows past the end are read from row S-1 and never stored, keys past the
@@ -329,7 +339,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     const uint16_t *Qh, *Kh, *Vh;
     uint16_t *Oh;
     if (GENERAL) {
-        const int bi = bh / a.H, hi = bh - bi * a.H, hk = hi / (a.H / a.Hk);
+        // Query heads that share a K/V head: the list walks the K/V heads fastest (list position -> XCD is
+        // round robin, so with a multiple of eight K/V heads all query heads of one K/V head run on the XCD
+        // whose L2 holds that head's K and V) and the members of a group slowest.
+        const int bi = bh / a.H, r = bh - bi * a.H, group = a.H / a.Hk;
+        const int hk = group > 1 ? r % a.Hk : r, hi = group > 1 ? hk * group + r / a.Hk : r;
+        bh = bi * a.H + hi;         // from here on the real head index (logsumexp, ALiBi slope, dropout)
         Qh = a.Q + (size_t)bi * a.q_bs + (size_t)hi * a.q_hs;
         Kh = a.K + (size_t)bi * a.k_bs + (size_t)hk * a.k_hs;
         Vh = a.V + (size_t)bi * a.v_bs + (size_t)hk * a.v_hs;
@@ -358,9 +373,17 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     const int rows_in_block = S - q0 < BR ? S - q0 : BR;
     int t0, t1;                 // key tiles visited by the workgroup
-    fa_tile_range(S, kBlockKeys, a.L, a.R, q0, rows_in_block, &t0, &t1);
+    fa_tile_range(Sk, kBlockKeys, a.L, a.R, q0 + pos_off, rows_in_block, &t0, &t1);
     int my_lo = 1, my_hi = 0;   // key tiles with at least one visible pair for this wave (contiguous)
-    if (wave_live) fa_tile_range(S, kBlockKeys, a.L, a.R, qw, WR, &my_lo, &my_hi);
+    if (wave_live) fa_tile_range(Sk, kBlockKeys, a.L, a.R, qw + pos_off, WR, &my_lo, &my_hi);
+    if (n_splits > 1) {         // this item's share of the key tiles; may leave nothing
+        const int s_lo = split * a.tiles_per_split, s_hi = s_lo + a.tiles_per_split - 1;
+        t0 = t0 > s_lo ? t0 : s_lo;
+        t1 = t1 < s_hi ? t1 : s_hi;
+        my_lo = my_lo > s_lo ? my_lo : s_lo;
+        my_hi = my_hi < s_hi ? my_hi : s_hi;
+    }
+    const bool any_tile = !GENERAL || t0 <= t1;
 
     // per-lane LDS read addresses for stage 0; stage, key block and key slice are immediates
     uint32_t koff[KS];
@@ -390,19 +413,19 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // they land in their own LDS rows and are masked)
     auto ragged_source = [&](int tile, int i, int rs, bool is_k) __attribute__((always_inline)) {
         const int P = (i * NW + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
-        const int last = S - 1 - tile * kBlockKeys, src_row = row < last ? row : last;
+        const int last = Sk - 1 - tile * kBlockKeys, src_row = row < last ? row : last;
         return (uint32_t)(src_row * (rs * 2) + ((pos ^ (is_k ? k_swz<CPR>(row) : v_swz<CPR>(row))) << 4));
     };
     auto issue_k = [&](int tile, int stage) __attribute__((always_inline)) {
         const char *src = reinterpret_cast<const char *>(Kh) + (size_t)tile * (kBlockKeys * 2) * k_rs;
-        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > S;
+        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > Sk;
 #pragma unroll
         for (int i = 0; i < IPW; ++i)
             dma_16(src, ragged ? ragged_source(tile, i, k_rs, true) : gk[i], lds0 + stage * TILEB + (i * NW + wave) * 1024);
     };
     auto issue_v = [&](int tile, int stage) __attribute__((always_inline)) {
         const char *src = reinterpret_cast<const char *>(Vh) + (size_t)tile * (kBlockKeys * 2) * v_rs;
-        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > S;
+        const bool ragged = GENERAL && (tile + 1) * kBlockKeys > Sk;
 #pragma unroll
         for (int i = 0; i < IPW; ++i)
             dma_16(src, ragged ? ragged_source(tile, i, v_rs, false) : gv[i], lds0 + LDS_V + stage * TILEB + (i * NW + wave) * 1024);
@@ -410,8 +433,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // skip / edge / free classification of a key tile for this wave (GENERAL: a tile that reaches past the
     // end of the sequence is an edge tile)
     auto tile_class = [&](int tile) __attribute__((always_inline)) {
-        int cls = fa_tile_class(kBlockKeys, a.L, a.R, qw, WR, tile);
-        if (GENERAL && cls == 2 && (tile + 1) * kBlockKeys > S) cls = 1;
+        int cls = fa_tile_class(kBlockKeys, a.L, a.R, qw + pos_off, WR, tile);
+        if (GENERAL && cls == 2 && (tile + 1) * kBlockKeys > Sk) cls = 1;
         return cls;
     };
 
@@ -450,9 +473,9 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         const int kb0 = tile * kBlockKeys + 4 * half;
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
-            const int q = my_q + 32 * b;
+            const int q = my_q + 32 * b + pos_off;
             // last visible key of this query (GENERAL: the sequence may end inside the tile)
-            const int j_hi = (GENERAL && q + a.R > S - 1) ? S - 1 : q + a.R;
+            const int j_hi = (GENERAL && q + a.R > Sk - 1) ? Sk - 1 : q + a.R;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
@@ -466,7 +489,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             // signed distance of this lane's query to the lane's first key of the tile: exact in fp32
-            const float base = (float)(my_q + 32 * b - (tile * kBlockKeys + 4 * half));
+            const float base = (float)(my_q + 32 * b + pos_off - (tile * kBlockKeys + 4 * half));
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float k0 = (float)(8 * (r >> 2) + (r & 3));
@@ -550,7 +573,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int b = 0; b < RB; ++b)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)bh, (uint32_t)(my_q + 32 * b),
+                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)bh, (uint32_t)(my_q + 32 * b + pos_off),
                                           (uint32_t)(2 * (2 * tile + kb) + half));
     };
     auto dropped = [&](float e, int b, int kb, int r) __attribute__((always_inline)) {
@@ -654,6 +677,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
     };
 
+    if (any_tile) {             // (GENERAL: a split, or a block of rows that sees no key, may have no tile at all)
     // ---- prologue: K(t0) .. K(t0+LA-1) resident before the first iteration
     issue_k(t0, 0);
     if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
@@ -716,8 +740,19 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
 
-    // rows 0..31 of a causal head are written by faithful_first_rows below instead
-    const bool faithful = MASKED && a.R == 0 && q0 == 0;
+    }   // any_tile
+
+    // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
+    // split that holds their keys, the first one; the others see none of their keys and write empty partials)
+    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off == 0 && split == 0;
+    // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
+    // own keys), which fa_combine_splits merges.
+    float *o_part = nullptr, *lse_part = nullptr;
+    if (GENERAL && n_splits > 1) {
+        const size_t part = (size_t)split * a.BH + bh;
+        o_part = a.o_part + part * S * D;
+        lse_part = a.lse_part + part * S;
+    }
     if (wave_live) {
         // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides)
 #pragma unroll
@@ -727,7 +762,22 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             if (GENERAL && q >= S) continue;       // a row past the end of the sequence
             const float l_half = l_a[b] + l_b[b];
             const float l_tot = l_half + swap_halves(l_half);
-            const float inv = 1.0f / l_tot;
+            const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
+            const float inv = empty ? 0.0f : 1.0f / l_tot;
+            const float lse_row = empty ? -INFINITY
+                                        : m_run[b] * (ALIBI ? 0.69314718055994530942f : a.scale) + __builtin_logf(l_tot);
+            if (GENERAL && o_part != nullptr) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 w = {o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv, o[b][db][4 * g + 2] * inv,
+                                         o[b][db][4 * g + 3] * inv};
+                        *reinterpret_cast<f32x4 *>(o_part + (size_t)q * D + 32 * db + 8 * g + 4 * half) = w;
+                    }
+                if (half == 0) lse_part[q] = lse_row;
+                continue;
+            }
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -737,14 +787,13 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
                     *reinterpret_cast<u32x2 *>(Oh + (size_t)q * o_rs + 32 * db + 8 * g + 4 * half) = w;
                 }
-            if (a.lse != nullptr && half == 0)
-                a.lse[(size_t)bh * S + q] = m_run[b] * (ALIBI ? 0.69314718055994530942f : a.scale) + __builtin_logf(l_tot);
+            if (a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
         }
     }
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
-        faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr, S, a.L, a.scale,
-                                     slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale, a.seed_lo,
-                                     a.seed_hi, (uint32_t)bh, reinterpret_cast<float *>(smem));
+        faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
+                                     S, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
+                                     a.seed_lo, a.seed_hi, (uint32_t)bh, reinterpret_cast<float *>(smem));
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
     if (a.queue != nullptr && tid == 0) {
@@ -754,6 +803,42 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             for (int x = 0; x < 9; ++x) a.queue[x] = 0u;
         }
     }
+}
+
+// Merges the partial results of a launch with key splits: for every query row,
+//   LSE = log sum_s exp(LSE_s),  O = sum_s exp(LSE_s - LSE) * O_s
+// (a split that saw no key of the row has LSE_s = -inf and weight 0).  One thread per four output elements.
+template <bool BF16, int D>
+__global__ void __launch_bounds__(256) fa_combine_splits(const FaKernelArgs a)
+{
+    constexpr int TPR = D / 4;                    // threads per row
+    const long long row = (long long)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+    const int c4 = (threadIdx.x % TPR) * 4;
+    const long long n_rows = (long long)a.BH * a.S;
+    if (row >= n_rows) return;
+    const int bh = (int)(row / a.S), q = (int)(row % a.S);
+    float mx = -INFINITY;
+    for (int s = 0; s < a.n_splits; ++s) mx = fmaxf(mx, a.lse_part[(size_t)s * n_rows + row]);
+    float wsum = 0.0f;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (mx != -INFINITY) {
+        for (int s = 0; s < a.n_splits; ++s) {
+            const float w = __expf(a.lse_part[(size_t)s * n_rows + row] - mx);
+            if (w > 0.0f) {
+                const f32x4 o = *reinterpret_cast<const f32x4 *>(a.o_part + ((size_t)s * n_rows + row) * D + c4);
+                acc += o * w;
+                wsum += w;
+            }
+        }
+        acc *= 1.0f / wsum;
+    }
+    const int bi = bh / a.H, hi = bh - bi * a.H;
+    uint16_t *dst = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs + (size_t)q * a.o_rs + c4;
+    u32x2 w2;
+    w2[0] = Num<BF16>::pack2(acc[0], acc[1]);
+    w2[1] = Num<BF16>::pack2(acc[2], acc[3]);
+    *reinterpret_cast<u32x2 *>(dst) = w2;
+    if (a.lse != nullptr && c4 == 0) a.lse[row] = mx == -INFINITY ? -INFINITY : mx + __logf(wsum);
 }
 
 template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST>

@@ -29,6 +29,11 @@ struct FaKernelArgs {
     int q_rs, k_rs, v_rs, o_rs;                 // row (sequence position) strides
     long long q_bs, q_hs, k_bs, k_hs;           // batch and head strides
     long long v_bs, v_hs, o_bs, o_hs;
+    int Sk;              // keys per head (S is the number of queries); query i sits at key position i + Sk - S
+    int n_splits;        // > 1: every (head, query block) is n_splits consecutive work items, each over
+    int tiles_per_split; //      tiles_per_split key tiles, writing partial results:
+    float *o_part;       //      [n_splits][BH][S][D] fp32, normalised over the split's own keys
+    float *lse_part;     //      [n_splits][BH][S] fp32, -inf where the split saw no key of the row
     // --- used by the DROPOUT instantiations only
     unsigned drop_threshold;   // key kept iff its byte >= threshold; p = threshold / 256
     float drop_scale;          // 256 / (256 - threshold)

@@ -33,6 +33,11 @@ FA_HD void fa_tile_range(int S, int block_keys, int L, int R, int q_begin, int r
     if (lo_key < 0) lo_key = 0;
     int hi_key = q_begin + rows - 1 + R;
     if (hi_key > S - 1) hi_key = S - 1;
+    if (hi_key < lo_key) {      // no visible key at all (queries placed before the first key, or past the last)
+        *tile_lo = 1;
+        *tile_hi = 0;
+        return;
+    }
     *tile_lo = lo_key / block_keys;
     *tile_hi = hi_key / block_keys;
 }

@@ -36,8 +36,9 @@ enum {
     FA_ERR_DEVICE = -8,            /* a HIP runtime call failed; see fa_last_device_error()  */
     FA_ERR_NO_DEVICE = -9,         /* no gfx950 device is visible                            */
     FA_ERR_TOO_LARGE = -10,        /* B*N*S*d or the work-item count overflows the kernel's index range */
-    FA_ERR_LAYOUT = -11            /* a stride is not a multiple of 8 elements or too small, n_kv_heads does
+    FA_ERR_LAYOUT = -11,           /* a stride is not a multiple of 8 elements or too small, n_kv_heads does
                                       not divide N, or a tensor pointer is not 16-byte aligned */
+    FA_ERR_WORKSPACE = -12         /* split_num > 1 and the workspace is NULL, misaligned or too small */
 };
 
 enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
@@ -81,7 +82,10 @@ typedef struct fa_fwd_params {
     int window_size_left;     /* keys with i - j > left are masked;  < 0 = unbounded          */
     int window_size_right;    /* keys with j - i > right are masked; < 0 = unbounded          */
     const float *alibi_slopes_ptr; /* [N] device floats: score -= slope[h]*|i-j| (mask.h:21-26), or NULL */
-    int split_num;            /* unused, as in the reference (utils.h:164)                    */
+    int split_num;            /* dead in the reference (utils.h:164).  Here: > 1 splits the keys of every
+                                 (head, query block) into that many work items whose partial results a
+                                 second kernel merges (long keys, few queries: decoding); needs
+                                 `workspace`.  <= 1: one pass                                   */
     /* --- beyond mykernelParamType --- */
     int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                 */
     int is_causal;            /* keys with j > i are masked (mask.h:27-38)                    */
@@ -95,11 +99,24 @@ typedef struct fa_fwd_params {
     long long k_strides[3];   /* same for K ({0,0,0} = contiguous [B,n_kv_heads,S,d])                   */
     long long v_strides[3];
     long long o_strides[3];   /* same for O ({0,0,0} = contiguous [B,N,S,d]); L is always [B,N,S]       */
+    int S_kv;                 /* keys per head when it differs from the S queries (0 = S).  K and V are
+                                 [B, n_kv_heads, S_kv, d]; query i sits at key position i + S_kv - S (the
+                                 queries are the last S positions), which is what the causal and window
+                                 masks, the ALiBi distance and the dropout decision see.  Rows that see no
+                                 key get O = 0 and L = -inf                                              */
+    void *workspace;          /* device scratch for split_num > 1, at least fa_fwd_workspace_bytes()    */
+    unsigned long long workspace_bytes;
 } fa_fwd_params;
 
 /* Checks a parameter block without touching any device.  Returns FA_OK or the
  * first violated FA_ERR_*.  (Replaces the reference's abort/throw/assert paths.) */
 int fa_fwd_validate(const fa_fwd_params *p);
+
+/* Device scratch a call with these parameters needs (0 unless split_num > 1):
+ * splits * B * N * S * (d + 1) * 4 bytes of fp32 partial outputs and logsumexps. */
+unsigned long long fa_fwd_workspace_bytes(const fa_fwd_params *p);
+/* A split count that fills the device for these shapes (1 when the problem has enough work items anyway). */
+int fa_fwd_suggest_splits(const fa_fwd_params *p);
 
 /* Enqueues the forward pass on `stream` and returns without synchronising.
  * Allocates nothing; Q/K/V are read-only, O (and L when non-NULL) are
