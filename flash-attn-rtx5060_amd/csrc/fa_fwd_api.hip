@@ -183,6 +183,25 @@ int fa_dropout_keep(unsigned long long seed, long long bh, int i, int j, int thr
 namespace {
 int key_tiles(const fa_fwd_params *p) { return ((p->S_kv > 0 ? p->S_kv : p->S) + kBlockKeysHost - 1) / kBlockKeysHost; }
 // splits actually used: at most one per key tile
+// Query heads per K/V head packed into the rows of one work item (1 = not packed): when there are few
+// queries behind long keys (decoding), all query heads of a K/V head fit one 128-row workgroup and K and V
+// are then read once per group instead of once per query head.
+int packed_group(const fa_fwd_params *p)
+{
+    const int hk = p->n_kv_heads > 0 ? p->n_kv_heads : p->N;
+    if (hk <= 0 || hk >= p->N || p->N % hk != 0) return 1;
+    const int group = p->N / hk, sk = p->S_kv > 0 ? p->S_kv : p->S;
+    if (sk <= p->S) return 1;                                  // queries must sit behind earlier keys
+    if ((long long)group * p->S > 32LL * waves_for(p->B, p->N, p->S)) return 1;
+    return group;
+}
+// work items before key splits
+long long base_items(const fa_fwd_params *p)
+{
+    const int pack = packed_group(p);
+    if (pack > 1) return (long long)p->B * (p->N / pack);
+    return fa_sched_num_items(p->B, p->N, p->S, p->d);
+}
 int effective_splits(const fa_fwd_params *p)
 {
     if (p->split_num <= 1) return 1;
@@ -204,7 +223,7 @@ int fa_fwd_suggest_splits(const fa_fwd_params *p)
     if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0) return 1;
     // work items without splits against the workgroups the device keeps resident; split until the device is
     // filled about twice, with at least four key tiles (256 keys) per split
-    const long long items = fa_sched_num_items(p->B, p->N, p->S, p->d);
+    const long long items = base_items(p);
     const long long resident = (long long)kComputeUnits * (waves_for(p->B, p->N, p->S) == 8 ? 1 : 2);
     if (items >= resident) return 1;
     long long n = (2 * resident + items - 1) / items;
@@ -224,7 +243,7 @@ int fa_fwd_validate(const fa_fwd_params *p)
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
     if (p->S_kv < 0) return FA_ERR_BAD_SHAPE;
-    if (fa_sched_num_items(p->B, p->N, p->S, p->d) * effective_splits(p) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (base_items(p) * effective_splits(p) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
     if (effective_splits(p) > 1 && (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
                                     p->workspace_bytes < fa_fwd_workspace_bytes(p))) return FA_ERR_WORKSPACE;
     if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
@@ -264,6 +283,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.tiles_per_split = (key_tiles(p) + a.n_splits - 1) / a.n_splits;
     a.o_part = static_cast<float *>(p->workspace);
     a.lse_part = a.o_part != nullptr ? a.o_part + (size_t)a.n_splits * p->B * p->N * p->S * p->d : nullptr;
+    a.pack = packed_group(p);
     bool general = a.Hk != p->N || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
     {
         const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
@@ -286,7 +306,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     }
     const int waves = waves_for(p->B, p->N, p->S);
     const int block_rows = 32 * waves;
-    a.n_qblocks = (p->S + block_rows - 1) / block_rows;
+    a.n_qblocks = a.pack > 1 ? 1 : (p->S + block_rows - 1) / block_rows;
     const int s_max = a.Sk > p->S ? a.Sk : p->S;        // stands in for "unbounded"
     fa_mask_bounds(s_max, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
     // (a sequence that ends inside a 64-key tile needs the element mask on that tile, whatever the mask)
@@ -294,7 +314,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.descending = (a.L < s_max || a.R < s_max) ? 1 : 0;
     a.scale = p->softmax_scale;
     a.scale_log2e = p->softmax_scale * 1.44269504088896340736f;
-    a.n_items = (long long)a.BH * a.n_qblocks * a.n_splits;
+    a.n_items = (long long)(a.BH / a.pack) * a.n_qblocks * a.n_splits;
 
     // Dispatch mode launches one workgroup per item, in list order; the hardware hands them to CUs as these
     // free up, which is a longest-first greedy schedule.  Persistent mode launches one resident set of

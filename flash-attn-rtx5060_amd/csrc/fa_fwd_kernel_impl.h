@@ -326,7 +326,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // (GENERAL with key splits: consecutive list positions are the splits of one (head, query block))
     const int n_splits = GENERAL ? a.n_splits : 1;
     const int split = n_splits > 1 ? (int)(item % n_splits) : 0;
-    fa_item_decode(n_splits > 1 ? item / n_splits : item, a.BH, a.n_qblocks, a.descending, &bh, &qblock);
+    // (GENERAL, packed groups: an item is a (batch, K/V head); its rows are the queries of all query heads
+    // of that K/V head, head after head -- few queries against long keys read K and V once per group)
+    const int pack = GENERAL ? a.pack : 1;
+    fa_item_decode(n_splits > 1 ? item / n_splits : item, pack > 1 ? a.BH / pack : a.BH, a.n_qblocks, a.descending, &bh, &qblock);
     const int S = a.S;
     // GENERAL: Sk keys; query i sits at key position i + pos_off (the queries are the last S positions), which
     // is what masks, the ALiBi distance and the dropout decision see.
@@ -342,8 +345,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         // Query heads that share a K/V head: the list walks the K/V heads fastest (list position -> XCD is
         // round robin, so with a multiple of eight K/V heads all query heads of one K/V head run on the XCD
         // whose L2 holds that head's K and V) and the members of a group slowest.
-        const int bi = bh / a.H, r = bh - bi * a.H, group = a.H / a.Hk;
-        const int hk = group > 1 ? r % a.Hk : r, hi = group > 1 ? hk * group + r / a.Hk : r;
+        int bi, hk, hi;
+        if (pack > 1) {             // bh counts (batch, K/V head); hi is the first query head of the group
+            bi = bh / a.Hk; hk = bh - bi * a.Hk; hi = hk * pack;
+        } else {
+            const int r = bh % a.H, group = a.H / a.Hk;
+            bi = bh / a.H;
+            hk = group > 1 ? r % a.Hk : r;
+            hi = group > 1 ? hk * group + r / a.Hk : r;
+        }
         bh = bi * a.H + hi;         // from here on the real head index (logsumexp, ALiBi slope, dropout)
         Qh = a.Q + (size_t)bi * a.q_bs + (size_t)hi * a.q_hs;
         Kh = a.K + (size_t)bi * a.k_bs + (size_t)hk * a.k_hs;
@@ -359,7 +369,30 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     const int q0 = qblock * BR;
     const int qw = q0 + wave * WR;          // first query row of this wave
     const int my_q = qw + l32;              // query row of row block 0 on this lane; block b adds 32*b
-    const bool wave_live = qw < S;          // (not GENERAL: S is a multiple of 128, a live wave has all its rows)
+    const int n_rows = pack * S;            // rows of this (head | packed group)
+    const bool wave_live = qw < n_rows;     // (not GENERAL: S is a multiple of 128, a live wave has all its rows)
+    // Row block b of this lane: the query position inside its head, the head relative to `bh`, whether the row
+    // exists (a row that does not exist computes on a copy of the last row and stores nothing).
+    int row_pos[RB], row_head[RB];
+    bool row_ok[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        const int r = my_q + 32 * b;
+        row_ok[b] = !GENERAL || r < n_rows;
+        const int rc = row_ok[b] ? r : n_rows - 1;
+        row_head[b] = pack > 1 ? rc / S : 0;
+        row_pos[b] = pack > 1 ? rc - row_head[b] * S : rc;
+    }
+    // the query positions this wave covers, for tile ranges and tile classes: its 32 rows when they lie in one
+    // head, every position when they wrap from one head of a packed group into the next
+    int wave_pos0 = qw, wave_npos = WR, block_pos0 = q0;
+    if (pack > 1) {
+        const int last = qw + WR - 1 < n_rows - 1 ? qw + WR - 1 : n_rows - 1;
+        const bool one_head = wave_live && qw / S == last / S;
+        wave_pos0 = one_head ? qw % S : 0;
+        wave_npos = one_head ? last - qw + 1 : S;
+        block_pos0 = 0;
+    }
 
     // Q^T fragments: B operand, lane = (query l32, head-dim slice 8*half..+7 of each 16)
     u32x4 qf[RB][KS];
@@ -368,14 +401,14 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int s = 0; s < KS; ++s)
             qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(
-                                       Qh + (size_t)((GENERAL && my_q + 32 * b >= S) ? S - 1 : my_q + 32 * b) * q_rs + 16 * s + 8 * half)
+                                       Qh + (GENERAL ? (size_t)row_head[b] * a.q_hs : 0) + (size_t)row_pos[b] * q_rs + 16 * s + 8 * half)
                                  : u32x4{0, 0, 0, 0};
 
-    const int rows_in_block = S - q0 < BR ? S - q0 : BR;
+    const int rows_in_block = pack > 1 ? S : S - q0 < BR ? S - q0 : BR;
     int t0, t1;                 // key tiles visited by the workgroup
-    fa_tile_range(Sk, kBlockKeys, a.L, a.R, q0 + pos_off, rows_in_block, &t0, &t1);
+    fa_tile_range(Sk, kBlockKeys, a.L, a.R, block_pos0 + pos_off, rows_in_block, &t0, &t1);
     int my_lo = 1, my_hi = 0;   // key tiles with at least one visible pair for this wave (contiguous)
-    if (wave_live) fa_tile_range(Sk, kBlockKeys, a.L, a.R, qw + pos_off, WR, &my_lo, &my_hi);
+    if (wave_live) fa_tile_range(Sk, kBlockKeys, a.L, a.R, wave_pos0 + pos_off, wave_npos, &my_lo, &my_hi);
     if (n_splits > 1) {         // this item's share of the key tiles; may leave nothing
         const int s_lo = split * a.tiles_per_split, s_hi = s_lo + a.tiles_per_split - 1;
         t0 = t0 > s_lo ? t0 : s_lo;
@@ -433,7 +466,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // skip / edge / free classification of a key tile for this wave (GENERAL: a tile that reaches past the
     // end of the sequence is an edge tile)
     auto tile_class = [&](int tile) __attribute__((always_inline)) {
-        int cls = fa_tile_class(kBlockKeys, a.L, a.R, qw + pos_off, WR, tile);
+        int cls = fa_tile_class(kBlockKeys, a.L, a.R, wave_pos0 + pos_off, wave_npos, tile);
         if (GENERAL && cls == 2 && (tile + 1) * kBlockKeys > Sk) cls = 1;
         return cls;
     };
@@ -454,7 +487,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // reference point and the exponent work on those values with a factor of one.
     const float c = a.scale_log2e;
     const float cs = ALIBI ? 1.0f : c;
-    const float slope = ALIBI ? a.alibi[bh % a.H] : 0.0f;
+    // (one slope per head: per lane when the rows of a wave belong to several heads of a packed group)
+    const float slope = ALIBI ? a.alibi[bh % a.H + (GENERAL ? row_head[0] : 0)] : 0.0f;
     const float slope_l2 = slope * 1.44269504088896340736f;
     const float thresh = kRescaleLog2 / cs;
     uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
@@ -473,7 +507,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         const int kb0 = tile * kBlockKeys + 4 * half;
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
-            const int q = my_q + 32 * b + pos_off;
+            const int q = row_pos[b] + pos_off;
             // last visible key of this query (GENERAL: the sequence may end inside the tile)
             const int j_hi = (GENERAL && q + a.R > Sk - 1) ? Sk - 1 : q + a.R;
 #pragma unroll
@@ -489,7 +523,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             // signed distance of this lane's query to the lane's first key of the tile: exact in fp32
-            const float base = (float)(my_q + 32 * b + pos_off - (tile * kBlockKeys + 4 * half));
+            const float base = (float)(row_pos[b] + pos_off - (tile * kBlockKeys + 4 * half));
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float k0 = (float)(8 * (r >> 2) + (r & 3));
@@ -573,7 +607,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int b = 0; b < RB; ++b)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)bh, (uint32_t)(my_q + 32 * b + pos_off),
+                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)(bh + (GENERAL ? row_head[b] : 0)),
+                                          (uint32_t)(row_pos[b] + pos_off),
                                           (uint32_t)(2 * (2 * tile + kb) + half));
     };
     auto dropped = [&](float e, int b, int kb, int r) __attribute__((always_inline)) {
@@ -744,12 +779,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
-    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off == 0 && split == 0;
+    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off == 0 && split == 0 && pack == 1;
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
     // own keys), which fa_combine_splits merges.
     float *o_part = nullptr, *lse_part = nullptr;
     if (GENERAL && n_splits > 1) {
-        const size_t part = (size_t)split * a.BH + bh;
+        const size_t part = (size_t)split * a.BH + bh;       // (row_head rows further for the heads of a packed group)
         o_part = a.o_part + part * S * D;
         lse_part = a.lse_part + part * S;
     }
@@ -758,8 +793,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             if (faithful && wave == 0 && b == 0) continue;
-            const int q = my_q + 32 * b;
-            if (GENERAL && q >= S) continue;       // a row past the end of the sequence
+            // the row's index in its head's [S, ...] output, counted from head `bh` (packed groups: row_head
+            // heads further on; their logsumexp and partial rows follow at S per head, their O rows at o_hs)
+            const int q = GENERAL ? row_head[b] * S + row_pos[b] : my_q + 32 * b;
+            if (!row_ok[b]) continue;              // a row past the end
             const float l_half = l_a[b] + l_b[b];
             const float l_tot = l_half + swap_halves(l_half);
             const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
@@ -785,7 +822,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     u32x2 w;
                     w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
                     w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2 *>(Oh + (size_t)q * o_rs + 32 * db + 8 * g + 4 * half) = w;
+                    *reinterpret_cast<u32x2 *>(Oh + (GENERAL ? (size_t)row_head[b] * a.o_hs + (size_t)row_pos[b] * o_rs : (size_t)q * o_rs) +
+                                               32 * db + 8 * g + 4 * half) = w;
                 }
             if (a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
         }

@@ -34,6 +34,8 @@ struct FaKernelArgs {
     int tiles_per_split; //      tiles_per_split key tiles, writing partial results:
     float *o_part;       //      [n_splits][BH][S][D] fp32, normalised over the split's own keys
     float *lse_part;     //      [n_splits][BH][S] fp32, -inf where the split saw no key of the row
+    int pack;            // > 1: work items are (batch, K/V head) and their rows the queries of the `pack` query
+                         //      heads of that K/V head, head after head (n_qblocks is 1)
     // --- used by the DROPOUT instantiations only
     unsigned drop_threshold;   // key kept iff its byte >= threshold; p = threshold / 256
     float drop_scale;          // 256 / (256 - threshold)
