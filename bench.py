@@ -34,6 +34,72 @@ WORKLOADS = {
 }
 
 
+# Few queries behind long keys (decoding): HBM-bound, not part of the headline metric.
+DECODE_WORKLOADS = {
+    # name: (B, H, Hk, S, S_kv, D, seed)
+    "d1": (16, 32, 8, 1, 8192, 128, 41),       # grouped K/V heads
+    "d2": (4, 32, 32, 1, 32768, 128, 42),      # one K/V head per query head, long keys
+}
+PEAK_HBM_GBS = 8000.0
+
+
+def decode_bench(args):
+    """One JSON line for a decode workload: a step is one forward pass of S new queries per head against S_kv
+    keys through fa_fwd with key splits; the roofline is HBM (K and V read once, Q, O and logsumexp)."""
+    import numpy as np
+    import torch
+    from __graft_entry__ import load_package
+    from parity_util import TOL, errors, from_torch, make_inputs, to_torch
+    import oracle_binding as ob
+
+    fa = load_package()
+    fa.lib()
+    B, H, Hk, S, Skv, D, seed = DECODE_WORKLOADS[args.workload]
+    q, _, _ = make_inputs(fa, (B, H, S, D), 0, seed)
+    _, k, v = make_inputs(fa, (B, Hk, Skv, D), 0, seed + 100)
+    tq, tk, tv = (to_torch(x, 0) for x in (q, k, v))
+    out = torch.empty_like(tq)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+
+    def step():
+        fa.flash_attention_forward(tq, tk, tv, causal=True, out=out, lse=lse, splits="auto")
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gpu_ms = e0.elapsed_time(e1) / args.steps
+    algo_bytes = 2 * B * Hk * Skv * D * 2 + 2 * B * H * S * D * 2 + B * H * S * 4
+    # parity: the queries are the last S rows of the square S_kv problem (rows are independent)
+    rep = H // Hk
+    qpad = np.zeros((B, H, Skv, D), dtype=np.uint16)
+    qpad[:, :, Skv - S:, :] = q
+    heads = np.arange(0, B * H, max(1, (B * H) // 64))
+    rows = (heads[:, None] * Skv + (Skv - S) + np.arange(S)[None, :]).reshape(-1).astype(np.int64)
+    o_ref, lse_ref = ob.rows(qpad, np.repeat(k, rep, axis=1), np.repeat(v, rep, axis=1), rows, 0, None, True, -1, -1)
+    sel = (heads[:, None] * S + np.arange(S)[None, :]).reshape(-1)
+    err = errors(ob.to_f32(from_torch(out), 0).reshape(-1, D)[sel], ob.to_f32(o_ref, 0), lse.cpu().numpy().reshape(-1)[sel], lse_ref)
+    err["rows_checked"] = int(len(rows))
+    err["within_tolerance"] = bool(err["nonfinite"] == 0 and err["max_abs"] <= TOL[0]["max_abs"] and err["rel_l2"] <= TOL[0]["rel_l2"]
+                                   and err["lse_abs"] <= TOL[0]["lse_abs"])
+    print(json.dumps({
+        "metric": "attn decode, K/V + Q + O bytes per second, 1 GPU", "value": round(algo_bytes / (wall_ms * 1e-3) / 1e9, 1),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: fp16 B{B} H{H} (K/V heads {Hk}) S{S} S_kv{Skv} D{D} causal, key splits auto",
+                   "seed": seed, "algorithmic_bytes": algo_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (gpu_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(algo_bytes / (gpu_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None,
+                     "kernel_ms_avg": round(gpu_ms, 5)},
+        "parity": err}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,7 +107,7 @@ def main():
     # warm-up steps of a 1 ms kernel the timed region still runs through the ramp and reads about 5 % low)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline sample; 0 disables")
     ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
     ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2, 3), help="0 library default, 1 dispatch, 2 persistent snake, 3 persistent queue")
@@ -54,6 +120,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards by (batch, head) with no "
                  "communication, but no multi-GPU run is part of this benchmark)")
+
+    if args.workload in DECODE_WORKLOADS:
+        return decode_bench(args)
 
     import numpy as np
     import torch
