@@ -307,9 +307,23 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (tid == 0) {
             // own XCD's list first; when that is exhausted, help the others (this also makes the result
             // independent of how the hardware spreads the workgroups over the XCDs)
+            // (When the own list is exhausted, all eight counters are read in one round trip before any is
+            // updated: a workgroup that finds nothing left then pays for one read instead of eight updates in
+            // a row, on counters that every other leaving workgroup updates at the same time.)
             unsigned found = 0xffffffffu;
-            for (unsigned xo = 0; xo < 8u && found == 0xffffffffu; ++xo) {
-                const unsigned xq = (xcd + xo) & 7u;
+            const long long own = (long long)atomicAdd(&a.queue[xcd], 1u) * 8 + xcd;
+            if (own < a.n_items) found = (unsigned)own;
+            while (found == 0xffffffffu) {
+                unsigned cnt[8];
+#pragma unroll
+                for (unsigned xo = 1; xo < 8u; ++xo)
+                    cnt[xo] = __hip_atomic_load(&a.queue[(xcd + xo) & 7u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                unsigned pick = 8u;
+#pragma unroll
+                for (unsigned xo = 7; xo >= 1u; --xo)
+                    if ((long long)cnt[xo] * 8 + ((xcd + xo) & 7u) < a.n_items) pick = xo;
+                if (pick == 8u) break;
+                const unsigned xq = (xcd + pick) & 7u;
                 const long long cand = (long long)atomicAdd(&a.queue[xq], 1u) * 8 + xq;
                 if (cand < a.n_items) found = (unsigned)cand;
             }
