@@ -112,6 +112,9 @@ def main():
     ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
     ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2, 3), help="0 library default, 1 dispatch, 2 persistent snake, 3 persistent queue")
     ap.add_argument("--alibi", action="store_true", help="add the ALiBi bias with slopes 2^(-8/H*(h+1)) (not the headline metric)")
+    ap.add_argument("--sigma", type=float, default=None,
+                    help="override the standard deviation of the inputs (0 = all-zero tensors: the same instruction "
+                         "stream without data-dependent switching power; not the headline metric)")
     ap.add_argument("--dropout", type=float, default=0.0, help="dropout probability (not the headline metric), seed 48")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
@@ -132,6 +135,8 @@ def main():
     fa = load_package()
     fa.lib()    # raises if the HIP library is missing: there is no fallback path
     B, H, S, D, dtype, causal, wl, sigma, frac, mult, seed = WORKLOADS[args.workload]
+    if args.sigma is not None:
+        sigma = args.sigma
     shape = (B, H, S, D)
     q, k, v = make_inputs(fa, shape, dtype, seed, sigma, frac, mult)
     tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
