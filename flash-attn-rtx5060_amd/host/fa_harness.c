@@ -32,7 +32,7 @@
 typedef struct {
     int B, N, S, d, bf16, causal, wl, wr, iters, warmup, threads, lse, alibi;
     unsigned long long seed;
-    float sigma, scale;
+    float sigma, scale, dropout;
     double row_fraction;
     float row_mult;
     const char *dump;
@@ -108,6 +108,7 @@ int main(int argc, char **argv)
         else if (!strcmp(a, "--dump")) { NEED_VALUE(); c.dump = v; }
         else if (!strcmp(a, "--no-lse")) c.lse = 0;
         else if (!strcmp(a, "--alibi")) c.alibi = 1;
+        else if (!strcmp(a, "--dropout")) { NEED_VALUE(); c.dropout = (float)atof(v); }
         else { fprintf(stderr, "unknown argument %s\n", a); return 2; }
     }
     if (!scale_given && c.d > 0) c.scale = (float)(1.0 / sqrt((double)c.d));
@@ -146,6 +147,8 @@ int main(int argc, char **argv)
     p.window_size_left = c.wl; p.window_size_right = c.wr;
     p.dtype = c.bf16 ? FA_DTYPE_BF16 : FA_DTYPE_F16;
     p.is_causal = c.causal;
+    p.dropout_prob = c.dropout;      /* main.cu:26,30 (dropout, dropout_prob) ... */
+    p.seed = 48;                     /* ... with the seed main() gives its curand states, main.cu:93 */
     float *hs = NULL;
     void *ds = NULL;
     if (c.alibi) {      /* the slopes of main.cu:36-45: -2^(-8/N * (h+1)), copied to the device */
@@ -181,11 +184,11 @@ int main(int argc, char **argv)
         if (!isfinite(x)) ++bad;                      /* main.cu:149 rejects NaN/Inf the same way */
     }
     printf("{\"config\": \"%s\", \"device\": \"%s\", \"compute_units\": %d, \"B\": %d, \"N\": %d, \"S\": %d, \"d\": %d, "
-           "\"dtype\": \"%s\", \"causal\": %d, \"window_left\": %d, \"window_right\": %d, \"alibi\": %d, \"scale\": %.9g, \"seed\": %llu, "
+           "\"dtype\": \"%s\", \"causal\": %d, \"window_left\": %d, \"window_right\": %d, \"alibi\": %d, \"dropout\": %.6g, \"scale\": %.9g, \"seed\": %llu, "
            "\"iters\": %d, \"ms_median\": %.6f, \"ms_min\": %.6f, \"algorithmic_flops\": %.6e, "
            "\"tflops_median\": %.3f, \"tflops_best\": %.3f, \"peak_tflops\": %.1f, \"frac_of_peak_median\": %.4f, "
            "\"nonfinite_outputs\": %zu}\n",
-           c.name, devname, cus, c.B, c.N, c.S, c.d, c.bf16 ? "bf16" : "fp16", c.causal, c.wl, c.wr, c.alibi, (double)c.scale,
+           c.name, devname, cus, c.B, c.N, c.S, c.d, c.bf16 ? "bf16" : "fp16", c.causal, c.wl, c.wr, c.alibi, (double)c.dropout, (double)c.scale,
            c.seed, c.iters, med, best, flops, flops / med / 1e9, flops / best / 1e9, PEAK_TFLOPS,
            flops / med / 1e9 / PEAK_TFLOPS, bad);
 

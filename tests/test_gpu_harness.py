@@ -18,6 +18,8 @@ pytestmark = pytest.mark.gpu
      (2, 3, 1024, 128), 1, True, 200, 5),
     (["--B", "1", "--N", "8", "--S", "1024", "--d", "64", "--causal", "--alibi", "--seed", "6"],
      (1, 8, 1024, 64), 0, True, -1, 6),
+    (["--B", "1", "--N", "4", "--S", "640", "--d", "128", "--causal", "--dropout", "0.1", "--seed", "8"],
+     (1, 4, 640, 128), 0, True, -1, 8),
 ])
 def test_harness_output_matches_oracle(fa, oracle, tmp_path, args, shape, dtype, causal, wl, seed):
     assert os.path.exists(fa.HARNESS_PATH), "fa_harness has not been built"
@@ -40,6 +42,7 @@ def test_harness_output_matches_oracle(fa, oracle, tmp_path, args, shape, dtype,
     if "--alibi" in args:       # the slopes of the reference's main() (src/main.cu:38-42)
         slopes = np.fromfile(f"{prefix}.slopes.bin", dtype=np.float32)
         assert np.array_equal(slopes, (-np.power(2.0, -8.0 / H * (np.arange(H) + 1))).astype(np.float32))
-    o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, causal, wl, -1, slopes)
+    drop = (fa.lib().fa_dropout_threshold(0.1), 48) if "--dropout" in args else (0, 0)   # seed 48: main.cu:93
+    o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, causal, wl, -1, slopes, dropout=drop)
     err = errors(oracle.to_f32(o[rows], dtype), oracle.to_f32(o_ref, dtype), lse[rows], lse_ref)
     assert_within(err, dtype, f"harness {args}")
