@@ -418,3 +418,90 @@ int fa_oracle_rows_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t
     }
     return bad ? -1 : 0;
 }
+
+/* ------------------------------------------------------------------ */
+/* gradients, fp64 (the reference has no backward pass: this is the     */
+/* mathematics of d/dQ, d/dK, d/dV of O = softmax(scale*Q*K^T + bias)*V */
+/* on the storage-type inputs, pinned by finite differences and by      */
+/* torch autograd in tests/test_oracle_bwd.py)                          */
+/* ------------------------------------------------------------------ */
+int fa_oracle_bwd_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                      const uint16_t *dO, double *dQ, double *dK, double *dV, int nthreads)
+{
+    if (!cfg_ok(c) || !Q || !K || !V || !dO || !dQ || !dK || !dV || c->dropout_threshold != 0) return -1;
+    const int S = c->S, D = c->D, dt = c->dtype;
+    const int64_t BH = (int64_t)c->B * c->H;
+    if (nthreads < 1) nthreads = 1;
+    double *lse = (double *)malloc((size_t)BH * S * sizeof(double));
+    double *delta = (double *)malloc((size_t)BH * S * sizeof(double));      /* D_i = dO_i . O_i */
+    if (!lse || !delta) { free(lse); free(delta); return -1; }
+    /* pass over query rows: logsumexp, D, dQ */
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 4)
+    for (int64_t row = 0; row < BH * S; ++row) {
+        const int64_t bh = row / S;
+        const int i = (int)(row % S);
+        const uint16_t *q = Q + (size_t)row * D, *k = K + (size_t)bh * S * D, *v = V + (size_t)bh * S * D, *g = dO + (size_t)row * D;
+        const double slope = c->alibi_slopes ? (double)c->alibi_slopes[bh % c->H] : 0.0;
+        int lo, hi; visible_range(c, i, &lo, &hi);
+        const int n = hi - lo + 1;
+        double *p = (double *)malloc(((size_t)(n > 0 ? n : 1) + 2 * (size_t)D) * sizeof(double));
+        double *o = p + (n > 0 ? n : 1), *dq = o + D;
+        double mx = -INFINITY;
+        for (int j = lo; j <= hi; ++j) {
+            double sc = 0.0;
+            for (int t = 0; t < D; ++t) sc += (double)widen(q[t], dt) * (double)widen(k[(size_t)j * D + t], dt);
+            sc = sc * (double)c->scale - slope * abs(i - j);
+            p[j - lo] = sc;
+            if (sc > mx) mx = sc;
+        }
+        double sum = 0.0;
+        for (int j = lo; j <= hi; ++j) { p[j - lo] = exp(p[j - lo] - mx); sum += p[j - lo]; }
+        for (int t = 0; t < D; ++t) { o[t] = 0.0; dq[t] = 0.0; }
+        for (int j = lo; j <= hi; ++j) {
+            p[j - lo] /= sum;
+            for (int t = 0; t < D; ++t) o[t] += p[j - lo] * (double)widen(v[(size_t)j * D + t], dt);
+        }
+        double dl = 0.0;
+        for (int t = 0; t < D; ++t) dl += (double)widen(g[t], dt) * o[t];
+        for (int j = lo; j <= hi; ++j) {
+            double dp = 0.0;
+            for (int t = 0; t < D; ++t) dp += (double)widen(g[t], dt) * (double)widen(v[(size_t)j * D + t], dt);
+            const double ds = p[j - lo] * (dp - dl) * (double)c->scale;
+            for (int t = 0; t < D; ++t) dq[t] += ds * (double)widen(k[(size_t)j * D + t], dt);
+        }
+        for (int t = 0; t < D; ++t) dQ[(size_t)row * D + t] = dq[t];
+        lse[row] = n > 0 ? mx + log(sum) : -INFINITY;
+        delta[row] = dl;
+        free(p);
+    }
+    /* pass over key rows: dK, dV from the stored logsumexp and D */
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 4)
+    for (int64_t row = 0; row < BH * S; ++row) {
+        const int64_t bh = row / S;
+        const int j = (int)(row % S);
+        const uint16_t *kj = K + (size_t)row * D, *vj = V + (size_t)row * D;
+        const uint16_t *q = Q + (size_t)bh * S * D, *g = dO + (size_t)bh * S * D;
+        const double slope = c->alibi_slopes ? (double)c->alibi_slopes[bh % c->H] : 0.0;
+        double *acc = (double *)calloc(2 * (size_t)D, sizeof(double));
+        double *dk = acc, *dv = acc + D;
+        for (int i = 0; i < S; ++i) {
+            if (masked(c, i, j)) continue;
+            double sc = 0.0, dp = 0.0;
+            for (int t = 0; t < D; ++t) {
+                sc += (double)widen(q[(size_t)i * D + t], dt) * (double)widen(kj[t], dt);
+                dp += (double)widen(g[(size_t)i * D + t], dt) * (double)widen(vj[t], dt);
+            }
+            sc = sc * (double)c->scale - slope * abs(i - j);
+            const double pij = exp(sc - lse[bh * S + i]);
+            const double ds = pij * (dp - delta[bh * S + i]) * (double)c->scale;
+            for (int t = 0; t < D; ++t) {
+                dk[t] += ds * (double)widen(q[(size_t)i * D + t], dt);
+                dv[t] += pij * (double)widen(g[(size_t)i * D + t], dt);
+            }
+        }
+        for (int t = 0; t < D; ++t) { dK[(size_t)row * D + t] = dk[t]; dV[(size_t)row * D + t] = dv[t]; }
+        free(acc);
+    }
+    free(lse); free(delta);
+    return 0;
+}

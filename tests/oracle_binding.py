@@ -38,6 +38,7 @@ def lib(scalar=False):
         L.fa_oracle_full.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp, vp, ctypes.c_int]
         L.fa_oracle_rows_f64.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp, ctypes.c_int64, vp, vp, ctypes.c_int]
         L.fa_oracle_literal.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp]
+        L.fa_oracle_bwd_f64.argtypes = [ctypes.POINTER(Cfg), vp, vp, vp, vp, vp, vp, vp, ctypes.c_int]
         L.fa_oracle_dropout_keep.argtypes = [ctypes.c_uint64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         L.fa_oracle_philox4x32_10.restype = None
         L.fa_oracle_philox4x32_10.argtypes = [ctypes.POINTER(ctypes.c_uint32)] * 3
@@ -108,6 +109,19 @@ def literal(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=N
     rc = lib(scalar).fa_oracle_literal(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data)
     assert rc == 0
     return o
+
+
+def bwd_f64(q, k, v, do, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None):
+    """fp64 gradients (dQ, dK, dV), each [B,H,S,D] float64, of sum(dO * O)."""
+    _check((q, k, v, do))
+    B, H, S, D = q.shape
+    scale = np.float32(1.0 / np.sqrt(D)) if scale is None else np.float32(scale)
+    dq, dk, dv = (np.empty((B, H, S, D), dtype=np.float64) for _ in range(3))
+    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes)
+    rc = lib().fa_oracle_bwd_f64(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, do.ctypes.data,
+                                 dq.ctypes.data, dk.ctypes.data, dv.ctypes.data, threads or default_threads())
+    assert rc == 0
+    return dq, dk, dv
 
 
 def to_f32(bits, dtype):
