@@ -48,6 +48,7 @@ EXPORTED_SYMBOLS = (
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
+    "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_algorithmic_flops",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
     "fa_event_elapsed_ms", "fa_event_destroy",
@@ -70,6 +71,20 @@ class FaFwdParams(ctypes.Structure):
         ("q_strides", ctypes.c_longlong * 3), ("k_strides", ctypes.c_longlong * 3),
         ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
         ("S_kv", ctypes.c_int), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_ulonglong),
+    ]
+
+
+class FaBwdParams(ctypes.Structure):
+    """struct fa_bwd_params of include/fa_bwd.h (field-for-field)."""
+    _fields_ = [
+        ("Q", ctypes.c_void_p), ("K", ctypes.c_void_p), ("V", ctypes.c_void_p), ("O", ctypes.c_void_p),
+        ("dO", ctypes.c_void_p), ("L", ctypes.c_void_p),
+        ("dQ", ctypes.c_void_p), ("dK", ctypes.c_void_p), ("dV", ctypes.c_void_p),
+        ("B", ctypes.c_int), ("N", ctypes.c_int), ("S", ctypes.c_int), ("d", ctypes.c_int),
+        ("softmax_scale", ctypes.c_float),
+        ("window_size_left", ctypes.c_int), ("window_size_right", ctypes.c_int),
+        ("dtype", ctypes.c_int), ("is_causal", ctypes.c_int),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_ulonglong),
     ]
 
 
@@ -122,6 +137,12 @@ def lib():
         L.fa_algorithmic_flops.restype = ctypes.c_double
         L.fa_algorithmic_flops.argtypes = [ctypes.c_int] * 7
         L.fa_dropout_threshold.argtypes = [ctypes.c_float]
+        L.fa_bwd_validate.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd.argtypes = [ctypes.POINTER(FaBwdParams), ctypes.c_void_p]
+        L.fa_bwd_workspace_bytes.restype = ctypes.c_ulonglong
+        L.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd_algorithmic_flops.restype = ctypes.c_double
+        L.fa_bwd_algorithmic_flops.argtypes = [ctypes.c_int] * 7
         L.fa_dropout_keep.argtypes = [ctypes.c_ulonglong, ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
@@ -223,6 +244,46 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
     if st != FA_OK:
         raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
     return (out, lse) if return_lse else out
+
+
+def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, lse_ptr=0, dq_ptr=0, dk_ptr=0, dv_ptr=0,
+                    softmax_scale=None, causal=False, window_left=-1, window_right=-1, dtype=FA_DTYPE_F16,
+                    workspace_ptr=0, workspace_bytes=0):
+    p = FaBwdParams()
+    p.Q, p.K, p.V, p.O, p.dO, p.L = q_ptr, k_ptr, v_ptr, o_ptr, do_ptr, lse_ptr
+    p.dQ, p.dK, p.dV = dq_ptr, dk_ptr, dv_ptr
+    p.B, p.N, p.S, p.d = B, N, S, d
+    p.softmax_scale = softmax_scale if softmax_scale is not None else (1.0 / math.sqrt(d) if d > 0 else 0.0)
+    p.window_size_left, p.window_size_right = window_left, window_right
+    p.dtype, p.is_causal = dtype, int(causal)
+    p.workspace, p.workspace_bytes = workspace_ptr, workspace_bytes
+    return p
+
+
+def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1):
+    """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
+    fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v and mask.  All tensors
+    contiguous [B, N, S, d] (lse [B, N, S] float32), S a multiple of 128, d 64 or 128."""
+    import torch
+    ts = (q, k, v, o, do)
+    if not all(t.is_cuda and t.is_contiguous() and t.dtype == q.dtype and t.shape == q.shape for t in ts):
+        raise ValueError("q, k, v, o, do must be contiguous GPU tensors of one shape and dtype")
+    if q.dtype not in (torch.float16, torch.bfloat16) or q.dim() != 4:
+        raise ValueError("tensors must be [B, N, S, d] float16 or bfloat16")
+    B, N, S, d = q.shape
+    if not (lse.is_cuda and lse.dtype == torch.float32 and lse.is_contiguous() and tuple(lse.shape) == (B, N, S)):
+        raise ValueError("lse must be a contiguous float32 GPU tensor [B, N, S]")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    p = make_bwd_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                        lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), softmax_scale, causal,
+                        window_left, window_right, FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16)
+    need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    p.workspace, p.workspace_bytes = workspace.data_ptr(), need
+    st = lib().fa_bwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream))
+    if st != FA_OK:
+        raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
+    return dq, dk, dv
 
 
 def run_flash_attention(B, N, S, d, Q, K, V, O, L=None, M=None, Is_dropout=False, Is_causal=False, Is_local=False,

@@ -14,6 +14,8 @@
 #include <mutex>
 
 #include "fa_fwd.h"
+#include "fa_bwd.h"
+#include "fa_bwd_args.h"
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
@@ -24,6 +26,7 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
+hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -82,8 +85,8 @@ const char *fa_strerror(int status)
     case FA_ERR_NULL_POINTER: return "Q, K, V or O is NULL";
     case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FA_ERR_SEQLEN_MULTIPLE: return "reserved (seqlen no longer has to be a multiple of 128)";
-    case FA_ERR_WORKSPACE: return "split_num > 1 needs a 16-byte aligned workspace of fa_fwd_workspace_bytes() bytes";
+    case FA_ERR_SEQLEN_MULTIPLE: return "the backward pass needs seqlen to be a multiple of 128";
+    case FA_ERR_WORKSPACE: return "needs a 16-byte aligned workspace of fa_fwd_workspace_bytes() (split_num > 1) or fa_bwd_workspace_bytes() bytes";
     case FA_ERR_LAYOUT: return "strides must be multiples of 8 elements (row strides at least head_dim), n_kv_heads must divide heads, pointers must be 16-byte aligned";
     case FA_ERR_UNSUPPORTED: return "dropout_prob must be at least 0 and below 1";
     case FA_ERR_DTYPE: return "dtype must be FA_DTYPE_F16 or FA_DTYPE_BF16";
@@ -431,5 +434,60 @@ int fa_event_elapsed_ms(void *start, void *stop, float *ms)
     return FA_OK;
 }
 int fa_event_destroy(void *ev) { FA_DEV(hipEventDestroy(static_cast<hipEvent_t>(ev)), "hipEventDestroy"); return FA_OK; }
+
+// ---- backward pass (include/fa_bwd.h); the reference has none ----
+
+
+unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
+{
+    if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0) return 0;
+    return (unsigned long long)p->B * p->N * p->S * 4ull;
+}
+
+int fa_bwd_validate(const fa_bwd_params *p)
+{
+    if (!p || !p->Q || !p->K || !p->V || !p->O || !p->dO || !p->L || !p->dQ || !p->dK || !p->dV) return FA_ERR_NULL_POINTER;
+    if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
+    if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
+    if (p->S % 128 != 0) return FA_ERR_SEQLEN_MULTIPLE;
+    if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
+    if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
+    if ((long long)p->B * p->N * (p->S / 128) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    const void *ptrs[8] = {p->Q, p->K, p->V, p->O, p->dO, p->dQ, p->dK, p->dV};
+    for (int t = 0; t < 8; ++t)
+        if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0) return FA_ERR_LAYOUT;
+    if (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
+        p->workspace_bytes < fa_bwd_workspace_bytes(p)) return FA_ERR_WORKSPACE;
+    return FA_OK;
+}
+
+int fa_bwd(const fa_bwd_params *p, void *stream)
+{
+    const int st = fa_bwd_validate(p);
+    if (st != FA_OK) return st;
+    FaBwdArgs a;
+    a.Q = static_cast<const uint16_t *>(p->Q);
+    a.K = static_cast<const uint16_t *>(p->K);
+    a.V = static_cast<const uint16_t *>(p->V);
+    a.O = static_cast<const uint16_t *>(p->O);
+    a.dO = static_cast<const uint16_t *>(p->dO);
+    a.lse = p->L;
+    a.delta = static_cast<float *>(p->workspace);
+    a.dQ = static_cast<uint16_t *>(p->dQ);
+    a.dK = static_cast<uint16_t *>(p->dK);
+    a.dV = static_cast<uint16_t *>(p->dV);
+    a.BH = p->B * p->N;
+    a.S = p->S;
+    fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
+    a.scale = p->softmax_scale;
+    const int masked = (a.L < p->S || a.R < p->S) ? 1 : 0;
+    hipError_t e = fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
+}
+
+double fa_bwd_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
+{
+    return 2.5 * fa_algorithmic_flops(B, N, S, d, is_causal, window_left, window_right);
+}
 
 }  // extern "C"

@@ -1,4 +1,4 @@
-"""C-ABI boundary without a GPU: the library loads, exports every symbol include/fa_fwd.h declares, and
+"""C-ABI boundary without a GPU: the library loads, exports every symbol include/*.h declares, and
 rejects bad arguments with status codes (the reference exits/aborts/throws: utils.h:16-23,
 flash_forward.h:384-387,587-589)."""
 import ctypes
@@ -13,7 +13,7 @@ REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_functions():
-    text = open(os.path.join(REPO, "include", "fa_fwd.h")).read()
+    text = "".join(open(os.path.join(REPO, "include", h)).read() for h in ("fa_fwd.h", "fa_bwd.h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"^\s*(?:const\s+)?(?:int|void|unsigned long long|long long|double|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
     return sorted(set(names))
@@ -50,6 +50,56 @@ def test_struct_layout_matches_header(fa):
     # the first twenty are mykernelParamType's, in its order (include/utils.h:143-165)
     assert fields[:20] == ["Q", "K", "V", "O", "L", "M", "B", "N", "S", "d", "Tr", "Tc", "softmax_scale", "dropout_prob",
                            "seed", "states", "window_size_left", "window_size_right", "alibi_slopes_ptr", "split_num"]
+
+
+def test_backward_struct_layout_and_status_codes(fa):
+    text = open(os.path.join(REPO, "include", "fa_bwd.h")).read()
+    body = re.search(r"typedef struct fa_bwd_params \{(.*?)\} fa_bwd_params;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for line in body.splitlines():
+        if ";" in line:
+            decl = line.split(";")[0]
+            fields += [re.sub(r"[\s\*]", "", part).split()[-1] if i else re.findall(r"(\w+)\s*$", part)[0]
+                       for i, part in enumerate(decl.split(","))]
+    assert fields == [f[0] for f in fa.FaBwdParams._fields_]
+    import subprocess
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "layout.c")
+        with open(src, "w") as f:
+            f.write('#include <stdio.h>\n#include <stddef.h>\n#include "fa_bwd.h"\n'
+                    'int main(void){printf("%zu %zu %zu\\n", sizeof(fa_bwd_params), offsetof(fa_bwd_params, softmax_scale),'
+                    ' offsetof(fa_bwd_params, workspace_bytes));return 0;}\n')
+        exe = os.path.join(tmp, "layout")
+        subprocess.run(["gcc", "-I", os.path.join(REPO, "include"), src, "-o", exe], check=True)
+        size, off_scale, off_ws = (int(x) for x in subprocess.run([exe], check=True, stdout=subprocess.PIPE, text=True).stdout.split())
+    assert size == ctypes.sizeof(fa.FaBwdParams)
+    assert off_scale == fa.FaBwdParams.softmax_scale.offset and off_ws == fa.FaBwdParams.workspace_bytes.offset
+
+    L = fa.lib()
+    ok = dict(B=2, N=4, S=1024, d=128, q_ptr=0x1000, k_ptr=0x2000, v_ptr=0x3000, o_ptr=0x4000, do_ptr=0x5000,
+              lse_ptr=0x6000, dq_ptr=0x7000, dk_ptr=0x8000, dv_ptr=0x9000, workspace_ptr=0xA000, workspace_bytes=2 * 4 * 1024 * 4)
+
+    def status(**kw):
+        a = dict(ok)
+        a.update(kw)
+        return L.fa_bwd_validate(ctypes.byref(fa.make_bwd_params(**a)))
+    assert status() == fa.FA_OK
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == 2 * 4 * 1024 * 4
+    assert L.fa_bwd_validate(None) == fa.FA_ERR_NULL_POINTER
+    for missing in ("q_ptr", "k_ptr", "v_ptr", "o_ptr", "do_ptr", "lse_ptr", "dq_ptr", "dk_ptr", "dv_ptr"):
+        assert status(**{missing: 0}) == fa.FA_ERR_NULL_POINTER
+    assert status(B=0) == fa.FA_ERR_BAD_SHAPE and status(S=-128) == fa.FA_ERR_BAD_SHAPE
+    assert status(d=96) == fa.FA_ERR_HEAD_DIM
+    assert status(S=1000) == fa.FA_ERR_SEQLEN_MULTIPLE
+    assert status(dtype=7) == fa.FA_ERR_DTYPE
+    assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE and status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE
+    assert status(dq_ptr=0x7008) == fa.FA_ERR_LAYOUT
+    assert status(workspace_ptr=0) == fa.FA_ERR_WORKSPACE and status(workspace_bytes=2 * 4 * 1024 * 4 - 1) == fa.FA_ERR_WORKSPACE
+    # launching needs a device; without one the call fails with a status, it does not crash
+    assert L.fa_bwd(ctypes.byref(fa.make_bwd_params(**dict(ok, S=1000))), None) == fa.FA_ERR_SEQLEN_MULTIPLE
+    assert L.fa_bwd_algorithmic_flops(2, 4, 1024, 128, 0, -1, -1) == 2.5 * L.fa_algorithmic_flops(2, 4, 1024, 128, 0, -1, -1)
 
 
 def test_validate_status_codes(fa):
