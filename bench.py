@@ -100,6 +100,68 @@ def decode_bench(args):
         "parity": err}))
 
 
+def backward_bench(args):
+    """One JSON line for the backward pass (fa_bwd: row sums, dQ, then dK and dV) on a forward workload's shape:
+    a step is one backward pass over the whole batch; FLOPs are 2.5 x the forward's (five products over the
+    unmasked pairs instead of two).  Parity: one head against torch's fp32 attention and autograd on the GPU
+    (the fp64 gradient oracle checks small shapes in tests/)."""
+    import numpy as np
+    import torch
+    from __graft_entry__ import load_package
+    from parity_util import make_inputs, to_torch
+
+    fa = load_package()
+    fa.lib()
+    B, H, S, D, dtype, causal, wl, sigma, frac, mult, seed = WORKLOADS[args.workload]
+    q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed, sigma, frac, mult)
+    do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed + 1000)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl)
+    grads = [None]
+
+    def step():
+        grads[0] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gpu_ms = e0.elapsed_time(e1) / args.steps
+    flops = fa.lib().fa_bwd_algorithmic_flops(B, H, S, D, int(causal), wl, -1)
+    # parity on the last head
+    qf, kf, vf = (t[-1, -1].float().requires_grad_(True) for t in (tq, tk, tv))
+    i = torch.arange(S, device="cuda")
+    vis = torch.ones((S, S), dtype=torch.bool, device="cuda")
+    if causal:
+        vis &= i[None, :] <= i[:, None]
+    if wl >= 0:
+        vis &= i[:, None] - i[None, :] <= wl
+    sc = (qf @ kf.T) * float(np.float32(1.0 / np.sqrt(D)))
+    (torch.softmax(sc.masked_fill(~vis, float("-inf")), dim=-1) @ vf).backward(tdo[-1, -1].float())
+    err = {}
+    for name, got, want in zip(("dQ", "dK", "dV"), grads[0], (qf.grad, kf.grad, vf.grad)):
+        d = got[-1, -1].float() - want
+        err[name] = {"rel_l2": float(d.norm() / want.norm()), "max_abs": float(d.abs().max()), "max_ref": float(want.abs().max())}
+    tf = flops / (wall_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "attn backward TFLOPS (dQ, dK, dV), 1 GPU", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
+        "config": {"workload": f"{args.workload} backward: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D}"
+                               f"{' causal' if causal else ''}{f' window_left {wl}' if wl >= 0 else ''}",
+                   "seed": seed, "algorithmic_flops": flops},
+        "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_delta + fa_bwd_dq + fa_bwd_dkdv"},
+        "parity_vs_torch_fp32_one_head": err}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +178,7 @@ def main():
                     help="override the standard deviation of the inputs (0 = all-zero tensors: the same instruction "
                          "stream without data-dependent switching power; not the headline metric)")
     ap.add_argument("--dropout", type=float, default=0.0, help="dropout probability (not the headline metric), seed 48")
+    ap.add_argument("--backward", action="store_true", help="time the backward pass on the workload's shape (not the headline metric)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters to bytes)")
@@ -126,6 +189,8 @@ def main():
 
     if args.workload in DECODE_WORKLOADS:
         return decode_bench(args)
+    if args.backward:
+        return backward_bench(args)
 
     import numpy as np
     import torch

@@ -132,8 +132,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 1) fa_bwd_dq(const FaBwdArgs a
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int S = a.S;
     const int n_qblocks = S / 128;
-    const int bh = (int)blockIdx.x / n_qblocks;
-    const int rank = (int)blockIdx.x % n_qblocks, qblock = MASKED ? n_qblocks - 1 - rank : rank;   // long blocks first
+    // one head per XCD at a time, long blocks first: the workgroups that share a head's K and V share an L2
+    int bh, qblock;
+    fa_item_decode((long long)blockIdx.x, a.BH, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
     const size_t head_off = (size_t)bh * S * D;
     const uint16_t *Qh = a.Q + head_off, *Kh = a.K + head_off, *Vh = a.V + head_off, *dOh = a.dO + head_off;
     const int q0 = qblock * 128, qw = q0 + wave * 32, my_q = qw + l32;
@@ -245,7 +246,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 1) fa_bwd_dkdv(const FaBwdArgs
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int S = a.S;
     const int n_kblocks = S / 128;
-    const int bh = (int)blockIdx.x / n_kblocks, kblock = (int)blockIdx.x % n_kblocks;
+    // one head per XCD at a time; key block 0 is seen by the most queries and goes first
+    int bh, kblock;
+    fa_item_decode((long long)blockIdx.x, a.BH, n_kblocks, 0, &bh, &kblock);
     const size_t head_off = (size_t)bh * S * D;
     const uint16_t *Qh = a.Q + head_off, *Kh = a.K + head_off, *Vh = a.V + head_off, *dOh = a.dO + head_off;
     const float *lse_h = a.lse + (size_t)bh * S, *delta_h = a.delta + (size_t)bh * S;
@@ -284,14 +287,16 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 1) fa_bwd_dkdv(const FaBwdArgs
         for (int r = 0; r < 16; ++r) { dk[db][r] = 0.0f; dv[db][r] = 0.0f; }
 
     if (t0 <= t1) {
-        issue(t0, 0);
+        // from the last query tile down to the diagonal: every workgroup of a head then starts on the same tile
+        // and the ones that run together keep reading the same tiles out of L2
+        issue(t1, 0);
         wait_vm<0>();
 #pragma unroll
         for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
-        for (int t = t0; t <= t1; ++t) {
-            const int stage = (t - t0) & 1;
-            if (t + 1 <= t1) {
-                issue(t + 1, stage ^ 1);
+        for (int t = t1; t >= t0; --t) {
+            const int stage = (t1 - t) & 1;
+            if (t - 1 >= t0) {
+                issue(t - 1, stage ^ 1);
                 if (wave < 2) wait_vm<4 * IPW + 1>(); else wait_vm<4 * IPW>();
             } else wait_vm<0>();
             phase_barrier();
