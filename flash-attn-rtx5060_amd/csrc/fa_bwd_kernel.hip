@@ -8,14 +8,14 @@
 //   dS = P o (dP - delta)
 //   dQ = scale * dS K,   dK = scale * dS^T Q
 //
-// Three kernels: fa_bwd_delta (one row per thread), fa_bwd_dq (a workgroup owns 128 queries and walks the key
-// tiles) and fa_bwd_dkdv (a workgroup owns 128 keys and walks the query tiles); no atomics, every output
-// element has one writer.  Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the
-// thing a wave owns on the lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B
+// Two kernels: fa_bwd_dq (a workgroup owns 256 queries and walks the key tiles; it also writes delta) and
+// fa_bwd_dkdv (a workgroup owns 256 keys and walks the query tiles); no atomics, every output element has one
+// writer, results are the same bits from run to run.
+// Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B
 // operands loaded once into registers, the walked tiles are A operands streamed through LDS by direct
 // global->LDS loads, and an accumulator tile is already laid out as the B operand of the next product.
-// A walked tile that is needed both row-wise (ds_read_b128) and transposed (ds_read_b64_tr_b16) is put into
-// LDS twice, once in each of the two bank-conflict-free swizzles.
+// A walked tile that is needed both row-wise (ds_read_b128) and transposed (ds_read_b64_tr_b16) sits in LDS
+// once, under a swizzle that is bank-conflict-free for both.
 #include "fa_fwd_kernel_impl.h"
 #include "fa_bwd_args.h"
 
@@ -121,30 +121,6 @@ __device__ __forceinline__ f32x16 zero16()
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// delta_i = sum_t dO_it * O_it, fp32 [B,H,S]
-// ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D>
-__global__ void __launch_bounds__(256) fa_bwd_delta(const FaBwdArgs a)
-{
-    const long long row = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (row >= (long long)a.BH * a.S) return;
-    const u32x4 *o = reinterpret_cast<const u32x4 *>(a.O + (size_t)row * D);
-    const u32x4 *g = reinterpret_cast<const u32x4 *>(a.dO + (size_t)row * D);
-    float sum = 0.0f;
-#pragma unroll
-    for (int c = 0; c < D / 8; ++c) {
-        const u32x4 x = o[c], y = g[c];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t xw = x[w], yw = y[w];
-            sum += storage_to_f32<BF16>((uint16_t)(xw & 0xffffu)) * storage_to_f32<BF16>((uint16_t)(yw & 0xffffu));
-            sum += storage_to_f32<BF16>((uint16_t)(xw >> 16)) * storage_to_f32<BF16>((uint16_t)(yw >> 16));
-        }
-    }
-    a.delta[row] = sum;
-}
-
-// ---------------------------------------------------------------------------------------------------------
 // dQ: a workgroup owns 256 queries (lane = query), walks the key tiles of its visible range.
 // LDS stage: K (read row-wise for S^T = K Q^T and transposed for dQ^T += K^T dS^T), V (row-wise, dP^T = V dO^T).
 // ---------------------------------------------------------------------------------------------------------
@@ -177,7 +153,24 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
         gf[s] = *reinterpret_cast<const u32x4 *>(dOh + (size_t)my_q * D + 16 * s + 8 * half);
     }
     float lse_l2 = a.lse[(size_t)bh * S + my_q] * kLog2e;
-    float delta = a.delta[(size_t)bh * S + my_q];
+    // delta_i = sum_t dO_it O_it: this lane holds half of row i of dO already; the other half is on lane ^ 32.
+    // Written out for fa_bwd_dkdv, which runs after this kernel.
+    float delta = 0.0f;
+    {
+        const uint16_t *Oh = a.O + head_off;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const u32x4 o = *reinterpret_cast<const u32x4 *>(Oh + (size_t)my_q * D + 16 * s + 8 * half);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t ow = o[w], gw = gf[s][w];
+                delta += storage_to_f32<BF16>((uint16_t)(ow & 0xffffu)) * storage_to_f32<BF16>((uint16_t)(gw & 0xffffu));
+                delta += storage_to_f32<BF16>((uint16_t)(ow >> 16)) * storage_to_f32<BF16>((uint16_t)(gw >> 16));
+            }
+        }
+        delta += swap_halves(delta);
+        if (active && half == 0) a.delta[(size_t)bh * S + my_q] = delta;
+    }
     const float c = a.scale * kLog2e;
 
     int t0, t1, my_lo = 1, my_hi = 0;
@@ -424,8 +417,6 @@ template <bool BF16, int D, bool MASKED>
 hipError_t launch_bwd(const FaBwdArgs &a, hipStream_t stream)
 {
     constexpr int TILEB = 64 * D * 2;
-    const long long rows = (long long)a.BH * a.S;
-    hipLaunchKernelGGL((fa_bwd_delta<BF16, D>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, a);
     const unsigned grid = (unsigned)((long long)a.BH * ((a.S + 255) / 256));
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512);
     auto kq = fa_bwd_dq<BF16, D, MASKED>;

@@ -35,7 +35,8 @@ typedef struct fa_bwd_params {
 
 int fa_bwd_validate(const fa_bwd_params *p);
 unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p);
-/* Enqueues three kernels on `stream` (row sums of dO*O, dQ, then dK and dV) and returns without synchronising. */
+/* Enqueues two kernels on `stream` (dQ and the row sums of dO*O, then dK and dV) and returns without
+ * synchronising.  No atomics: the same inputs give the same bits on every run. */
 int fa_bwd(const fa_bwd_params *p, void *stream);
 /* Algorithmic FLOPs of the backward pass: 10 * B * N * d * pairs (five products over the unmasked pairs). */
 double fa_bwd_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right);
