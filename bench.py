@@ -101,7 +101,7 @@ def decode_bench(args):
 
 
 def backward_bench(args):
-    """One JSON line for the backward pass (fa_bwd: row sums, dQ, then dK and dV) on a forward workload's shape:
+    """One JSON line for the backward pass (fa_bwd: dQ with the row sums of dO*O, then dK and dV) on a forward workload's shape:
     a step is one backward pass over the whole batch; FLOPs are 2.5 x the forward's (five products over the
     unmasked pairs instead of two).  Parity: one head against torch's fp32 attention and autograd on the GPU
     (the fp64 gradient oracle checks small shapes in tests/)."""
@@ -158,7 +158,7 @@ def backward_bench(args):
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_delta + fa_bwd_dq + fa_bwd_dkdv"},
+                     "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_dq + fa_bwd_dkdv"},
         "parity_vs_torch_fp32_one_head": err}))
 
 
