@@ -85,6 +85,11 @@ class FaBwdParams(ctypes.Structure):
         ("window_size_left", ctypes.c_int), ("window_size_right", ctypes.c_int),
         ("dtype", ctypes.c_int), ("is_causal", ctypes.c_int),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_ulonglong),
+        ("n_kv_heads", ctypes.c_int), ("S_kv", ctypes.c_int), ("alibi_slopes_ptr", ctypes.c_void_p),
+        ("q_strides", ctypes.c_longlong * 3), ("k_strides", ctypes.c_longlong * 3),
+        ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
+        ("do_strides", ctypes.c_longlong * 3), ("dq_strides", ctypes.c_longlong * 3),
+        ("dk_strides", ctypes.c_longlong * 3), ("dv_strides", ctypes.c_longlong * 3),
     ]
 
 
@@ -248,7 +253,8 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
 
 def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, lse_ptr=0, dq_ptr=0, dk_ptr=0, dv_ptr=0,
                     softmax_scale=None, causal=False, window_left=-1, window_right=-1, dtype=FA_DTYPE_F16,
-                    workspace_ptr=0, workspace_bytes=0):
+                    workspace_ptr=0, workspace_bytes=0, n_kv_heads=0, S_kv=0, alibi_ptr=0, strides=None):
+    """strides: dict name -> (batch, head, row) element strides for any of q, k, v, o, do, dq, dk, dv."""
     p = FaBwdParams()
     p.Q, p.K, p.V, p.O, p.dO, p.L = q_ptr, k_ptr, v_ptr, o_ptr, do_ptr, lse_ptr
     p.dQ, p.dK, p.dV = dq_ptr, dk_ptr, dv_ptr
@@ -257,26 +263,45 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
     p.window_size_left, p.window_size_right = window_left, window_right
     p.dtype, p.is_causal = dtype, int(causal)
     p.workspace, p.workspace_bytes = workspace_ptr, workspace_bytes
+    p.n_kv_heads, p.S_kv, p.alibi_slopes_ptr = n_kv_heads, S_kv, alibi_ptr
+    for name, st in (strides or {}).items():
+        if st is not None:
+            getattr(p, name + "_strides")[:] = list(st)
     return p
 
 
-def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1):
+def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
+                             alibi_slopes=None):
     """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
-    fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v and mask.  All tensors
-    contiguous [B, N, S, d] (lse [B, N, S] float32), S a multiple of 128, d 64 or 128."""
+    fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask and slopes.
+    Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
+    [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
     import torch
-    ts = (q, k, v, o, do)
-    if not all(t.is_cuda and t.is_contiguous() and t.dtype == q.dtype and t.shape == q.shape for t in ts):
-        raise ValueError("q, k, v, o, do must be contiguous GPU tensors of one shape and dtype")
-    if q.dtype not in (torch.float16, torch.bfloat16) or q.dim() != 4:
-        raise ValueError("tensors must be [B, N, S, d] float16 or bfloat16")
+    if not all(t.is_cuda and t.dtype == q.dtype and t.dim() == 4 and t.stride(3) == 1 for t in (q, k, v, o, do)):
+        raise ValueError("q, k, v, o, do must be 4-d GPU tensors of one dtype with a contiguous head dimension")
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("tensors must be float16 or bfloat16")
+    if o.shape != q.shape or do.shape != q.shape or k.shape != v.shape or (q.shape[0], q.shape[3]) != (
+            k.shape[0], k.shape[3]) or k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0 or k.shape[2] == 0:
+        raise ValueError("q, o, do must be [B, N, S, d], k and v [B, Nk, S_kv, d] with Nk dividing N")
     B, N, S, d = q.shape
+    Nk, S_kv = k.shape[1], k.shape[2]
     if not (lse.is_cuda and lse.dtype == torch.float32 and lse.is_contiguous() and tuple(lse.shape) == (B, N, S)):
         raise ValueError("lse must be a contiguous float32 GPU tensor [B, N, S]")
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
+                                         and alibi_slopes.is_contiguous() and tuple(alibi_slopes.shape) == (N,)):
+        raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)        # keep the inputs' strides
+    for t in (dq, dk, dv):
+        if t.stride(3) != 1:
+            raise ValueError("q, k, v must be laid out so that empty_like keeps a contiguous head dimension")
+    tensors = dict(q=q, k=k, v=v, o=o, do=do, dq=dq, dk=dk, dv=dv)
+    strides = {n: (None if t.is_contiguous() else tuple(t.stride()[:3])) for n, t in tensors.items()}
     p = make_bwd_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                         lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), softmax_scale, causal,
-                        window_left, window_right, FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16)
+                        window_left, window_right, FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16,
+                        n_kv_heads=0 if Nk == N else Nk, S_kv=0 if S_kv == S else S_kv,
+                        alibi_ptr=0 if alibi_slopes is None else alibi_slopes.data_ptr(), strides=strides)
     need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
     workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), need

@@ -3,13 +3,23 @@
 #define FA_BWD_ARGS_H
 #include <stdint.h>
 
+// One tensor [B, heads, rows, D] with a contiguous last dimension: element strides of the other three.
+struct FaBwdTensor {
+    long long bs, hs;
+    int rs;
+};
+
 struct FaBwdArgs {
-    const uint16_t *Q, *K, *V, *O, *dO;     // contiguous [B,H,S,D]
-    const float *lse;                       // [B,H,S], natural log, as the forward pass writes it
-    float *delta;                           // [B,H,S] scratch: sum_t dO*O per row
-    uint16_t *dQ, *dK, *dV;                 // contiguous [B,H,S,D]
-    int BH, S;
-    int L, R;                               // key j visible to query i iff i - L <= j <= i + R
+    const uint16_t *Q, *K, *V, *O, *dO;
+    const float *lse;                       // [B,H,S] contiguous, natural log, as the forward pass writes it
+    float *delta;                           // [B,H,S] scratch: sum_t dO*O per row, written by fa_bwd_dq
+    float *lse2;                            // [B,H,S] scratch: lse * log2(e), +inf for rows that saw no key
+    uint16_t *dQ, *dK, *dV;
+    const float *alibi;                     // [H] slopes or NULL
+    FaBwdTensor q, k, v, o, dO_, dq, dk, dv;
+    int B, H, Hk;                           // query heads, K/V heads (Hk divides H)
+    int S, Sk;                              // queries, keys; query i sits at key position i + Sk - S
+    int L, R;                               // key j visible to the query at position p iff p - L <= j <= p + R
     float scale;
 };
 

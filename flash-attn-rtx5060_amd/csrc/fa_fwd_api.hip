@@ -26,7 +26,7 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
-hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, hipStream_t stream);
+hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -85,7 +85,7 @@ const char *fa_strerror(int status)
     case FA_ERR_NULL_POINTER: return "Q, K, V or O is NULL";
     case FA_ERR_BAD_SHAPE: return "batch, heads and seqlen must be positive";
     case FA_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FA_ERR_SEQLEN_MULTIPLE: return "the backward pass needs seqlen to be a multiple of 128";
+    case FA_ERR_SEQLEN_MULTIPLE: return "reserved (seqlen no longer has to be a multiple of 128)";
     case FA_ERR_WORKSPACE: return "needs a 16-byte aligned workspace of fa_fwd_workspace_bytes() (split_num > 1) or fa_bwd_workspace_bytes() bytes";
     case FA_ERR_LAYOUT: return "strides must be multiples of 8 elements (row strides at least head_dim), n_kv_heads must divide heads, pointers must be 16-byte aligned";
     case FA_ERR_UNSUPPORTED: return "dropout_prob must be at least 0 and below 1";
@@ -436,26 +436,35 @@ int fa_event_elapsed_ms(void *start, void *stop, float *ms)
 int fa_event_destroy(void *ev) { FA_DEV(hipEventDestroy(static_cast<hipEvent_t>(ev)), "hipEventDestroy"); return FA_OK; }
 
 // ---- backward pass (include/fa_bwd.h); the reference has none ----
-
-
 unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
 {
     if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0) return 0;
-    return (unsigned long long)p->B * p->N * p->S * 4ull;
+    return 2ull * (unsigned long long)p->B * p->N * p->S * 4ull;       // delta and the rescaled logsumexp
 }
 
 int fa_bwd_validate(const fa_bwd_params *p)
 {
     if (!p || !p->Q || !p->K || !p->V || !p->O || !p->dO || !p->L || !p->dQ || !p->dK || !p->dV) return FA_ERR_NULL_POINTER;
-    if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
+    if (p->B <= 0 || p->N <= 0 || p->S <= 0 || p->S_kv < 0) return FA_ERR_BAD_SHAPE;
     if (p->d != 64 && p->d != 128) return FA_ERR_HEAD_DIM;
-    if (p->S % 128 != 0) return FA_ERR_SEQLEN_MULTIPLE;
     if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
-    if ((long long)p->B * p->N * (p->S / 128) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
+    const long long s_kv = p->S_kv > 0 ? p->S_kv : p->S;
+    if ((long long)p->B * p->N * ((p->S + 255) / 256) > 0x7fffffffLL || (long long)p->B * p->N * ((s_kv + 255) / 256) > 0x7fffffffLL ||
+        (long long)p->S + s_kv > 0x3fffffffLL) return FA_ERR_TOO_LARGE;
     const void *ptrs[8] = {p->Q, p->K, p->V, p->O, p->dO, p->dQ, p->dK, p->dV};
-    for (int t = 0; t < 8; ++t)
+    const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
+                                   p->dq_strides, p->dk_strides, p->dv_strides};
+    for (int t = 0; t < 8; ++t) {
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0) return FA_ERR_LAYOUT;
+        const long long *st = strides[t];
+        if (st[0] == 0 && st[1] == 0 && st[2] == 0) continue;       // contiguous
+        for (int k = 0; k < 3; ++k)
+            if (st[k] < 0 || st[k] % 8 != 0) return FA_ERR_LAYOUT;
+        if (st[2] < p->d) return FA_ERR_LAYOUT;
+        if (st[2] > (1LL << 24)) return FA_ERR_TOO_LARGE;           // per-lane byte offsets inside a tile are 32-bit
+    }
     if (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
         p->workspace_bytes < fa_bwd_workspace_bytes(p)) return FA_ERR_WORKSPACE;
     return FA_OK;
@@ -473,18 +482,46 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.dO = static_cast<const uint16_t *>(p->dO);
     a.lse = p->L;
     a.delta = static_cast<float *>(p->workspace);
+    a.lse2 = a.delta + (size_t)p->B * p->N * p->S;
     a.dQ = static_cast<uint16_t *>(p->dQ);
     a.dK = static_cast<uint16_t *>(p->dK);
     a.dV = static_cast<uint16_t *>(p->dV);
-    a.BH = p->B * p->N;
+    a.alibi = p->alibi_slopes_ptr;
+    a.B = p->B;
+    a.H = p->N;
+    a.Hk = p->n_kv_heads > 0 ? p->n_kv_heads : p->N;
     a.S = p->S;
-    fa_mask_bounds(p->S, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
+    a.Sk = p->S_kv > 0 ? p->S_kv : p->S;
+    bool general = a.Hk != a.H || a.S % 128 != 0 || a.Sk != a.S || a.alibi != nullptr;
+    {
+        const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
+                                       p->dq_strides, p->dk_strides, p->dv_strides};
+        FaBwdTensor *out[8] = {&a.q, &a.k, &a.v, &a.o, &a.dO_, &a.dq, &a.dk, &a.dv};
+        for (int t = 0; t < 8; ++t) {
+            const bool kv = t == 1 || t == 2 || t == 6 || t == 7;
+            const long long heads = kv ? a.Hk : a.H, len = kv ? a.Sk : a.S;
+            const long long dense[3] = {heads * len * p->d, len * p->d, p->d};
+            const long long *st = strides[t];
+            const bool given = st[0] != 0 || st[1] != 0 || st[2] != 0;
+            long long eff[3];
+            for (int k = 0; k < 3; ++k) {
+                eff[k] = given ? st[k] : dense[k];
+                if (eff[k] != dense[k]) general = true;
+            }
+            out[t]->bs = eff[0]; out[t]->hs = eff[1]; out[t]->rs = (int)eff[2];
+        }
+    }
+    // "unbounded" must stay unbounded after the shift by Sk - S that the key-owning kernel applies
+    const int far = a.S + a.Sk;
+    fa_mask_bounds(far, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
     a.scale = p->softmax_scale;
-    const int masked = (a.L < p->S || a.R < p->S) ? 1 : 0;
-    hipError_t e = fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, static_cast<hipStream_t>(stream));
+    const int masked = (general || a.L < far || a.R < far) ? 1 : 0;
+    hipError_t e = fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general ? 1 : 0, a.alibi != nullptr ? 1 : 0,
+                                      static_cast<hipStream_t>(stream));
     return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
 }
 
+// Five products over the unmasked pairs (the forward has two).  Square problems only, like fa_algorithmic_flops.
 double fa_bwd_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
 {
     return 2.5 * fa_algorithmic_flops(B, N, S, d, is_causal, window_left, window_right);

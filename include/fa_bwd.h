@@ -6,9 +6,10 @@
  * written (reference src/flash_forward.h:602,628-644).  This is the consumer of the logsumexp this library
  * adds.  Same C ABI conventions as fa_fwd.h: plain pointers and ints, an int status, nothing is allocated.
  *
- * Supported: the reference's layout only, contiguous [B,N,S,d] fp16 or bf16 with S a multiple of 128 and d 64
- * or 128; causal and one- or two-sided window masks.  Not in the parameter block, hence not supported: ALiBi, dropout, strides, grouped K/V heads;
- * other lengths are refused with FA_ERR_SEQLEN_MULTIPLE.
+ * Layouts as in fa_fwd(): fp16 or bf16, d 64 or 128, any S >= 1, contiguous [B,N,S,d] or element strides with a
+ * contiguous last dimension, K/V with n_kv_heads heads (dK and dV are summed over the query heads of a group) and
+ * S_kv keys (query i sits at key position i + S_kv - S), causal and one- or two-sided window masks, ALiBi.
+ * Not in the parameter block, hence not supported: dropout, key splits.
  */
 #ifndef FA_BWD_H
 #define FA_BWD_H
@@ -18,19 +19,31 @@ extern "C" {
 #endif
 
 typedef struct fa_bwd_params {
-    const void *Q, *K, *V;    /* [B,N,S,d] device, the forward inputs                                  */
-    const void *O;            /* [B,N,S,d] device, the forward output                                  */
-    const void *dO;           /* [B,N,S,d] device, gradient of the loss with respect to O              */
-    const float *L;           /* [B,N,S] fp32 logsumexp written by the forward pass                     */
-    void *dQ, *dK, *dV;       /* [B,N,S,d] device, fully overwritten, same type as the inputs           */
+    const void *Q, *K, *V;    /* device, the forward inputs: Q [B,N,S,d]; K, V [B,n_kv_heads,S_kv,d]              */
+    const void *O;            /* [B,N,S,d] device, the forward output                                          */
+    const void *dO;           /* [B,N,S,d] device, gradient of the loss with respect to O                      */
+    const float *L;           /* [B,N,S] contiguous fp32 logsumexp written by the forward pass                  */
+    void *dQ, *dK, *dV;       /* device, shaped like Q, K, V; fully overwritten, same type as the inputs        */
     int B, N, S, d;
     float softmax_scale;
-    int window_size_left;     /* as in fa_fwd_params                                                   */
+    int window_size_left;     /* as in fa_fwd_params                                                           */
     int window_size_right;
-    int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                          */
+    int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                                  */
     int is_causal;
-    void *workspace;          /* device scratch, at least fa_bwd_workspace_bytes(): B*N*S floats         */
+    void *workspace;          /* device scratch, at least fa_bwd_workspace_bytes(): 2*B*N*S floats               */
     unsigned long long workspace_bytes;
+    /* ---- general layouts; all zero = the reference's contiguous [B,N,S,d] with S_kv = S ---- */
+    int n_kv_heads;           /* 0 = N; otherwise divides N                                                    */
+    int S_kv;                 /* 0 = S                                                                         */
+    const float *alibi_slopes_ptr;   /* [N] fp32 device or NULL, as in fa_fwd_params                            */
+    long long q_strides[3];   /* element strides of (batch, head, row); {0,0,0} = contiguous                   */
+    long long k_strides[3];
+    long long v_strides[3];
+    long long o_strides[3];
+    long long do_strides[3];
+    long long dq_strides[3];
+    long long dk_strides[3];
+    long long dv_strides[3];
 } fa_bwd_params;
 
 int fa_bwd_validate(const fa_bwd_params *p);

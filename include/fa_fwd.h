@@ -28,8 +28,8 @@ enum {
     FA_ERR_NULL_POINTER = -1,      /* Q, K, V or O is NULL                                  */
     FA_ERR_BAD_SHAPE = -2,         /* B, N or S is not positive                              */
     FA_ERR_HEAD_DIM = -3,          /* d not in {64, 128}: reference throws, flash_forward.h:587 */
-    FA_ERR_SEQLEN_MULTIPLE = -4,   /* S % 128 != 0: fa_bwd() only (the reference assumes it silently,
-                                      :134,637); fa_fwd() accepts any S >= 1                */
+    FA_ERR_SEQLEN_MULTIPLE = -4,   /* reserved (was: S % 128 != 0, which the reference assumes silently,
+                                      :134,637); any S >= 1 is accepted now                 */
     FA_ERR_UNSUPPORTED = -5,       /* dropout_prob is not in [0, 1)                          */
     FA_ERR_DTYPE = -6,             /* dtype is neither FA_DTYPE_F16 nor FA_DTYPE_BF16        */
     FA_ERR_SCALE = -7,             /* softmax_scale is not a finite positive number          */

@@ -59,9 +59,8 @@ def test_backward_struct_layout_and_status_codes(fa):
     fields = []
     for line in body.splitlines():
         if ";" in line:
-            decl = line.split(";")[0]
-            fields += [re.sub(r"[\s\*]", "", part).split()[-1] if i else re.findall(r"(\w+)\s*$", part)[0]
-                       for i, part in enumerate(decl.split(","))]
+            decl = re.sub(r"\[\d+\]", "", line.split(";")[0])
+            fields += [re.findall(r"(\w+)\s*$", part)[0] for part in decl.split(",")]
     assert fields == [f[0] for f in fa.FaBwdParams._fields_]
     import subprocess
     import tempfile
@@ -70,35 +69,37 @@ def test_backward_struct_layout_and_status_codes(fa):
         with open(src, "w") as f:
             f.write('#include <stdio.h>\n#include <stddef.h>\n#include "fa_bwd.h"\n'
                     'int main(void){printf("%zu %zu %zu\\n", sizeof(fa_bwd_params), offsetof(fa_bwd_params, softmax_scale),'
-                    ' offsetof(fa_bwd_params, workspace_bytes));return 0;}\n')
+                    ' offsetof(fa_bwd_params, dv_strides));return 0;}\n')
         exe = os.path.join(tmp, "layout")
         subprocess.run(["gcc", "-I", os.path.join(REPO, "include"), src, "-o", exe], check=True)
         size, off_scale, off_ws = (int(x) for x in subprocess.run([exe], check=True, stdout=subprocess.PIPE, text=True).stdout.split())
     assert size == ctypes.sizeof(fa.FaBwdParams)
-    assert off_scale == fa.FaBwdParams.softmax_scale.offset and off_ws == fa.FaBwdParams.workspace_bytes.offset
+    assert off_scale == fa.FaBwdParams.softmax_scale.offset and off_ws == fa.FaBwdParams.dv_strides.offset
 
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128, q_ptr=0x1000, k_ptr=0x2000, v_ptr=0x3000, o_ptr=0x4000, do_ptr=0x5000,
-              lse_ptr=0x6000, dq_ptr=0x7000, dk_ptr=0x8000, dv_ptr=0x9000, workspace_ptr=0xA000, workspace_bytes=2 * 4 * 1024 * 4)
+              lse_ptr=0x6000, dq_ptr=0x7000, dk_ptr=0x8000, dv_ptr=0x9000, workspace_ptr=0xA000, workspace_bytes=2 * 2 * 4 * 1024 * 4)
 
     def status(**kw):
         a = dict(ok)
         a.update(kw)
         return L.fa_bwd_validate(ctypes.byref(fa.make_bwd_params(**a)))
     assert status() == fa.FA_OK
-    assert L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == 2 * 4 * 1024 * 4
+    assert L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == 2 * 2 * 4 * 1024 * 4
     assert L.fa_bwd_validate(None) == fa.FA_ERR_NULL_POINTER
     for missing in ("q_ptr", "k_ptr", "v_ptr", "o_ptr", "do_ptr", "lse_ptr", "dq_ptr", "dk_ptr", "dv_ptr"):
         assert status(**{missing: 0}) == fa.FA_ERR_NULL_POINTER
     assert status(B=0) == fa.FA_ERR_BAD_SHAPE and status(S=-128) == fa.FA_ERR_BAD_SHAPE
     assert status(d=96) == fa.FA_ERR_HEAD_DIM
-    assert status(S=1000) == fa.FA_ERR_SEQLEN_MULTIPLE
+    assert status(S=1000) == fa.FA_OK and status(S_kv=-1) == fa.FA_ERR_BAD_SHAPE
+    assert status(n_kv_heads=3) == fa.FA_ERR_LAYOUT and status(n_kv_heads=2) == fa.FA_OK
+    assert status(strides=dict(dk=(8, 8, 100))) == fa.FA_ERR_LAYOUT and status(strides=dict(q=(4 * 1024 * 256, 256, 4 * 256))) == fa.FA_OK
     assert status(dtype=7) == fa.FA_ERR_DTYPE
     assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE and status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE
     assert status(dq_ptr=0x7008) == fa.FA_ERR_LAYOUT
-    assert status(workspace_ptr=0) == fa.FA_ERR_WORKSPACE and status(workspace_bytes=2 * 4 * 1024 * 4 - 1) == fa.FA_ERR_WORKSPACE
+    assert status(workspace_ptr=0) == fa.FA_ERR_WORKSPACE and status(workspace_bytes=2 * 2 * 4 * 1024 * 4 - 1) == fa.FA_ERR_WORKSPACE
     # launching needs a device; without one the call fails with a status, it does not crash
-    assert L.fa_bwd(ctypes.byref(fa.make_bwd_params(**dict(ok, S=1000))), None) == fa.FA_ERR_SEQLEN_MULTIPLE
+    assert L.fa_bwd(ctypes.byref(fa.make_bwd_params(**dict(ok, d=80))), None) == fa.FA_ERR_HEAD_DIM
     assert L.fa_bwd_algorithmic_flops(2, 4, 1024, 128, 0, -1, -1) == 2.5 * L.fa_algorithmic_flops(2, 4, 1024, 128, 0, -1, -1)
 
 

@@ -85,13 +85,89 @@ def test_backward_refuses_what_it_does_not_cover(fa):
     L = fa.lib()
     ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
 
-    def params(S=128, d=64, ws_bytes=1024):
+    def params(S=128, d=64, ws_bytes=1024, **kw):
         ptr = t.data_ptr()
         return fa.make_bwd_params(1, 1, S, d, ptr, ptr, ptr, ptr, ptr, lse.data_ptr(), ptr, ptr, ptr,
-                                  workspace_ptr=ws.data_ptr(), workspace_bytes=ws_bytes)
+                                  workspace_ptr=ws.data_ptr(), workspace_bytes=ws_bytes, **kw)
     assert L.fa_bwd_validate(ctypes.byref(params())) == fa.FA_OK
-    assert L.fa_bwd(ctypes.byref(params(S=100)), None) == fa.FA_ERR_SEQLEN_MULTIPLE
     assert L.fa_bwd(ctypes.byref(params(d=96)), None) == fa.FA_ERR_HEAD_DIM
-    assert L.fa_bwd(ctypes.byref(params(ws_bytes=511)), None) == fa.FA_ERR_WORKSPACE
+    assert L.fa_bwd(ctypes.byref(params(ws_bytes=1023)), None) == fa.FA_ERR_WORKSPACE
+    assert L.fa_bwd(ctypes.byref(params(n_kv_heads=2)), None) == fa.FA_ERR_LAYOUT
+    assert L.fa_bwd(ctypes.byref(params(strides=dict(dq=(0, 0, 60)))), None) == fa.FA_ERR_LAYOUT
     p = params(); p.dK = 0
     assert L.fa_bwd(ctypes.byref(p), None) == fa.FA_ERR_NULL_POINTER
+
+def oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes):
+    """q, do [B,H,S,D], k, v [B,Hk,Skv,D] (storage bits) -> fp64 dq [B,H,S,D], dk, dv [B,Hk,Skv,D].
+    The oracle differentiates square problems with one K/V head per query head.  Grouped heads: repeat K and V
+    and sum their gradients over the group.  S < Skv: the queries are the last S rows of the square Skv problem
+    whose first rows carry dO = 0 (such a row contributes nothing to dK or dV and rows do not interact)."""
+    B, H, S, D = q.shape
+    Hk, Skv = k.shape[1], k.shape[2]
+    rep, off = H // Hk, Skv - S
+    assert off >= 0
+    kf, vf = (np.repeat(x, rep, axis=1) if rep > 1 else x for x in (k, v))
+    qpad = np.zeros((B, H, Skv, D), dtype=np.uint16)
+    dopad = np.zeros((B, H, Skv, D), dtype=np.uint16)
+    qpad[:, :, off:], dopad[:, :, off:] = q, do
+    dq, dk, dv = oracle.bwd_f64(qpad, kf, vf, dopad, dtype, None, causal, wl, wr, slopes)
+    return dq[:, :, off:], dk.reshape(B, Hk, rep, Skv, D).sum(axis=2), dv.reshape(B, Hk, rep, Skv, D).sum(axis=2)
+
+
+GENERAL = [
+    # B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd
+    (1, 2, 2, 100, 100, 64, 0, True, -1, -1, False, False),        # ragged length
+    (2, 4, 2, 333, 333, 128, 0, True, -1, -1, False, False),       # ... with grouped K/V heads
+    (1, 4, 1, 256, 256, 128, 0, False, -1, -1, False, True),       # one K/V head, [B,S,H,D] storage
+    (1, 2, 2, 200, 456, 128, 0, True, -1, -1, False, False),       # more keys than queries, causal
+    (1, 3, 3, 77, 300, 64, 1, False, -1, -1, False, True),         # cross attention, bf16
+    (1, 4, 2, 384, 384, 128, 0, True, -1, -1, True, False),        # ALiBi with grouped heads
+    (1, 2, 2, 190, 190, 64, 0, False, 50, 30, True, True),         # ALiBi, two-sided window, [B,S,H,D]
+    (1, 8, 2, 512, 640, 128, 1, True, 200, -1, False, True),
+    (1, 2, 2, 1, 500, 128, 0, True, -1, -1, False, False),         # a single query
+    (1, 2, 1, 300, 300, 128, 0, True, -1, -1, False, False),
+    (1, 2, 2, 256, 256, 64, 0, True, -1, -1, True, False),         # ALiBi on a shape the plain kernels cover
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,Skv,D,dtype,causal,wl,wr,alibi,bshd", GENERAL)
+def test_general_layouts_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd):
+    import torch
+    q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=700 + S)
+    do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=701 + S)
+    _, k, v = make_inputs(fa, (B, Hk, Skv, D), dtype, seed=702 + Skv)
+    slopes = (np.power(2.0, -8.0 / H * (np.arange(H) + 1)) * np.where(np.arange(H) % 2, -0.5, 1.0)).astype(np.float32) if alibi else None
+    dq_ref, dk_ref, dv_ref = oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    if bshd:
+        tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
+    ts = None if slopes is None else torch.from_numpy(slopes).cuda()
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, alibi_slopes=ts)
+    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, alibi_slopes=ts)
+    torch.cuda.synchronize()
+    assert dq.stride() == tq.stride() and dk.stride() == tk.stride() and dv.stride() == tv.stride()
+    for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
+        err = grad_errors(oracle.to_f32(from_torch(got.contiguous()), dtype), want)
+        print((B, H, Hk, S, Skv, D), dtype, causal, wl, wr, alibi, bshd, name, err, flush=True)
+        check(err, dtype, name)
+
+
+def test_queries_without_any_key_get_zero_gradients(fa):
+    """More queries than keys under a causal mask: the first S - S_kv queries see nothing (O = 0, logsumexp
+    -inf in the forward pass); their dQ is 0, they add nothing to dK and dV, and nothing is NaN."""
+    import torch
+    B, H, S, Skv, D = 1, 2, 192, 64, 64
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q, do = (torch.randn((B, H, S, D), device="cuda", generator=g).half() for _ in range(2))
+    k, v = (torch.randn((B, H, Skv, D), device="cuda", generator=g).half() for _ in range(2))
+    o, lse = fa.flash_attention_forward(q, k, v, causal=True)
+    dq, dk, dv = fa.flash_attention_backward(q, k, v, o, lse, do, causal=True)
+    torch.cuda.synchronize()
+    blind = S - Skv
+    assert bool((dq[:, :, :blind] == 0).all())
+    qf, kf, vf = (t.float().requires_grad_(True) for t in (q[:, :, blind:], k, v))
+    torch.nn.functional.scaled_dot_product_attention(qf, kf, vf, is_causal=True).backward(do[:, :, blind:].float())
+    for name, got, want in (("dQ", dq[:, :, blind:], qf.grad), ("dK", dk, kf.grad), ("dV", dv, vf.grad)):
+        err = grad_errors(got.float().cpu().numpy(), want.cpu().numpy())
+        print("blind rows", name, err, flush=True)
+        check(err, 0, name)
