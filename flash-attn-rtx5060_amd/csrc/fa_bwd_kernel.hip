@@ -106,9 +106,13 @@ template <int D> struct TileLoader {
     // a tile whose last rows lie past the end of the tensor: they are filled with copies of row `valid - 1`
     __device__ __forceinline__ void load_ragged(const uint16_t *tile_src, uint32_t lds_tile, int valid, int row_bytes) const
     {
+        // (the empty asm keeps the address arithmetic of this rare path inside its branch: hoisted out of the
+        // tile loop it would occupy registers for the whole kernel)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
-            const int P = (i * kBwdWaves + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
+            const int P = (i * kBwdWaves + wave) * 64 + ln, row = P / CPR, pos = P % CPR;
             const int src_row = row < valid ? row : valid - 1;
             dma_16(reinterpret_cast<const char *>(tile_src), (uint32_t)(src_row * row_bytes + ((pos ^ u_swz<CPR>(row)) << 4)),
                    lds_tile + (i * kBwdWaves + wave) * 1024);
@@ -391,8 +395,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             const int valid = S - tile * 64;
             ldq.load_ragged(Qh + (size_t)tile * 64 * q_rs, base, valid, q_rs * 2);
             ldg.load_ragged(dOh + (size_t)tile * 64 * g_rs, base + TILEB, valid, g_rs * 2);
-            if (wave == 0) dma_4(lse_h + tile * 64, lane < valid ? lane : valid - 1, base + 2 * TILEB);
-            if (wave == 1) dma_4(delta_h + tile * 64, lane < valid ? lane : valid - 1, base + 2 * TILEB + 256);
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            if (wave == 0) dma_4(lse_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB);
+            if (wave == 1) dma_4(delta_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB + 256);
         } else {
             ldq.load(Qh + (size_t)tile * 64 * q_rs, base);
             (GENERAL ? ldg : ldq).load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
