@@ -428,7 +428,9 @@ int fa_oracle_rows_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t
 int fa_oracle_bwd_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                       const uint16_t *dO, double *dQ, double *dK, double *dV, int nthreads)
 {
-    if (!cfg_ok(c) || !Q || !K || !V || !dO || !dQ || !dK || !dV || c->dropout_threshold != 0) return -1;
+    if (!cfg_ok(c) || !Q || !K || !V || !dO || !dQ || !dK || !dV) return -1;
+    /* dropout: O = sum_j m_ij p_ij v_j with m_ij = keep_ij / (1 - p); m enters dV and dP, the softmax Jacobian sees p */
+    const double keep_scale = 256.0 / (256.0 - (double)c->dropout_threshold);
     const int S = c->S, D = c->D, dt = c->dtype;
     const int64_t BH = (int64_t)c->B * c->H;
     if (nthreads < 1) nthreads = 1;
@@ -459,13 +461,17 @@ int fa_oracle_bwd_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t 
         for (int t = 0; t < D; ++t) { o[t] = 0.0; dq[t] = 0.0; }
         for (int j = lo; j <= hi; ++j) {
             p[j - lo] /= sum;
-            for (int t = 0; t < D; ++t) o[t] += p[j - lo] * (double)widen(v[(size_t)j * D + t], dt);
+            const double m = c->dropout_threshold == 0 ? 1.0
+                : fa_oracle_dropout_keep(c->dropout_seed, bh, i, j, c->dropout_threshold) ? keep_scale : 0.0;
+            for (int t = 0; t < D; ++t) o[t] += m * p[j - lo] * (double)widen(v[(size_t)j * D + t], dt);
         }
         double dl = 0.0;
         for (int t = 0; t < D; ++t) dl += (double)widen(g[t], dt) * o[t];
         for (int j = lo; j <= hi; ++j) {
             double dp = 0.0;
             for (int t = 0; t < D; ++t) dp += (double)widen(g[t], dt) * (double)widen(v[(size_t)j * D + t], dt);
+            if (c->dropout_threshold != 0)
+                dp *= fa_oracle_dropout_keep(c->dropout_seed, bh, i, j, c->dropout_threshold) ? keep_scale : 0.0;
             const double ds = p[j - lo] * (dp - dl) * (double)c->scale;
             for (int t = 0; t < D; ++t) dq[t] += ds * (double)widen(k[(size_t)j * D + t], dt);
         }
@@ -493,10 +499,12 @@ int fa_oracle_bwd_f64(const fa_oracle_cfg *c, const uint16_t *Q, const uint16_t 
             }
             sc = sc * (double)c->scale - slope * abs(i - j);
             const double pij = exp(sc - lse[bh * S + i]);
-            const double ds = pij * (dp - delta[bh * S + i]) * (double)c->scale;
+            const double m = c->dropout_threshold == 0 ? 1.0
+                : fa_oracle_dropout_keep(c->dropout_seed, bh, i, j, c->dropout_threshold) ? keep_scale : 0.0;
+            const double ds = pij * (m * dp - delta[bh * S + i]) * (double)c->scale;
             for (int t = 0; t < D; ++t) {
                 dk[t] += ds * (double)widen(q[(size_t)i * D + t], dt);
-                dv[t] += pij * (double)widen(g[(size_t)i * D + t], dt);
+                dv[t] += m * pij * (double)widen(g[(size_t)i * D + t], dt);
             }
         }
         for (int t = 0; t < D; ++t) { dK[(size_t)row * D + t] = dk[t]; dV[(size_t)row * D + t] = dv[t]; }

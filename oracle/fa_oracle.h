@@ -93,7 +93,8 @@ int fa_oracle_literal(const fa_oracle_cfg *cfg, const uint16_t *Q, const uint16_
  * Gradients of sum(dO * O) with respect to Q, K, V in fp64: dQ, dK, dV are [B,H,S,D] doubles.  The reference has
  * no backward pass; this is the textbook derivative (dV = P^T dO, dP = dO V^T, dS = P o (dP - rowsum(dO o O)),
  * dQ = scale dS K, dK = scale dS^T Q) on the storage-type inputs, with the same masks and ALiBi bias as the
- * forward functions; dropout is not supported (returns -1).
+ * forward functions and dropout decisions (O = sum_j m_ij p_ij v_j with m_ij = keep_ij / (1 - p): m scales dV's P and
+ * dP, the softmax Jacobian sees the undropped p).
  */
 int fa_oracle_bwd_f64(const fa_oracle_cfg *cfg, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                       const uint16_t *dO, double *dQ, double *dK, double *dV, int nthreads);

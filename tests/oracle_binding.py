@@ -111,13 +111,13 @@ def literal(q, k, v, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=N
     return o
 
 
-def bwd_f64(q, k, v, do, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None):
+def bwd_f64(q, k, v, do, dtype=F16, scale=None, causal=False, wl=-1, wr=-1, slopes=None, threads=None, dropout=(0, 0)):
     """fp64 gradients (dQ, dK, dV), each [B,H,S,D] float64, of sum(dO * O)."""
     _check((q, k, v, do))
     B, H, S, D = q.shape
     scale = np.float32(1.0 / np.sqrt(D)) if scale is None else np.float32(scale)
     dq, dk, dv = (np.empty((B, H, S, D), dtype=np.float64) for _ in range(3))
-    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes)
+    c = _cfg(q.shape, dtype, scale, causal, wl, wr, slopes, dropout)
     rc = lib().fa_oracle_bwd_f64(ctypes.byref(c), q.ctypes.data, k.ctypes.data, v.ctypes.data, do.ctypes.data,
                                  dq.ctypes.data, dk.ctypes.data, dv.ctypes.data, threads or default_threads())
     assert rc == 0

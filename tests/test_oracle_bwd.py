@@ -89,3 +89,31 @@ def test_structure_of_the_gradients():
     vconst = np.broadcast_to(v[:, :, :1, :], shape).copy()
     dq, dk, _ = ob.bwd_f64(q, k, vconst, do, F16, None, True)
     assert np.max(np.abs(dq)) <= 1e-12 and np.max(np.abs(dk)) <= 1e-12
+
+
+@pytest.mark.parametrize("dtype,causal,p", [(F16, False, 0.25), (F16, True, 0.5), (BF16, True, 0.1)])
+def test_dropout_gradients_against_torch_autograd_f64(dtype, causal, p):
+    """With dropout the output is sum_j m_ij p_ij v_j, m_ij = keep_ij / (1 - p).  The keep decisions come from
+    the numpy implementation of their published definition (parity_util.numpy_keep_mask), not from oracle code;
+    torch differentiates softmax -> mask -> matmul in fp64."""
+    import torch
+    from parity_util import numpy_keep_mask
+    rng = np.random.default_rng(33)
+    shape = (1, 3, 80, 32)
+    B, H, S, D = shape
+    thr, seed = int(round(p * 256)), 0x1234ABCD5678
+    q, k, v, do = (rand_bits(rng, shape, dtype) for _ in range(4))
+    dq, dk, dv = ob.bwd_f64(q, k, v, do, dtype, None, causal, -1, -1, None, dropout=(thr, seed))
+    tq, tk, tv, tdo = (torch.from_numpy(ob.to_f32(x, dtype).astype(np.float64)) for x in (q, k, v, do))
+    tq.requires_grad_(True); tk.requires_grad_(True); tv.requires_grad_(True)
+    i, j = np.meshgrid(np.arange(S), np.arange(S), indexing="ij")
+    bias = np.where((j <= i) if causal else np.ones((S, S), dtype=bool), 0.0, -np.inf)
+    keep = np.stack([numpy_keep_mask(seed, bh, S, thr) for bh in range(B * H)]).reshape(B, H, S, S)
+    m = torch.from_numpy(keep.astype(np.float64) * (256.0 / (256.0 - thr)))
+    s = torch.einsum("bhid,bhjd->bhij", tq, tk) * float(np.float32(1 / np.sqrt(D))) + torch.from_numpy(bias)
+    o = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, dim=-1) * m, tv)
+    (o * tdo).sum().backward()
+    assert 0.02 < 1.0 - keep.mean() < 0.98
+    assert np.allclose(dq, tq.grad.numpy(), atol=1e-11)
+    assert np.allclose(dk, tk.grad.numpy(), atol=1e-11)
+    assert np.allclose(dv, tv.grad.numpy(), atol=1e-11)
