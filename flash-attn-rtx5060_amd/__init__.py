@@ -90,6 +90,7 @@ class FaBwdParams(ctypes.Structure):
         ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
         ("do_strides", ctypes.c_longlong * 3), ("dq_strides", ctypes.c_longlong * 3),
         ("dk_strides", ctypes.c_longlong * 3), ("dv_strides", ctypes.c_longlong * 3),
+        ("dropout_prob", ctypes.c_float), ("seed", ctypes.c_ulonglong),
     ]
 
 
@@ -253,7 +254,8 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
 
 def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, lse_ptr=0, dq_ptr=0, dk_ptr=0, dv_ptr=0,
                     softmax_scale=None, causal=False, window_left=-1, window_right=-1, dtype=FA_DTYPE_F16,
-                    workspace_ptr=0, workspace_bytes=0, n_kv_heads=0, S_kv=0, alibi_ptr=0, strides=None):
+                    workspace_ptr=0, workspace_bytes=0, n_kv_heads=0, S_kv=0, alibi_ptr=0, strides=None, dropout_prob=0.0,
+                    seed=0):
     """strides: dict name -> (batch, head, row) element strides for any of q, k, v, o, do, dq, dk, dv."""
     p = FaBwdParams()
     p.Q, p.K, p.V, p.O, p.dO, p.L = q_ptr, k_ptr, v_ptr, o_ptr, do_ptr, lse_ptr
@@ -264,6 +266,7 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
     p.dtype, p.is_causal = dtype, int(causal)
     p.workspace, p.workspace_bytes = workspace_ptr, workspace_bytes
     p.n_kv_heads, p.S_kv, p.alibi_slopes_ptr = n_kv_heads, S_kv, alibi_ptr
+    p.dropout_prob, p.seed = dropout_prob, seed
     for name, st in (strides or {}).items():
         if st is not None:
             getattr(p, name + "_strides")[:] = list(st)
@@ -271,9 +274,10 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
 
 
 def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                             alibi_slopes=None):
+                             alibi_slopes=None, dropout_prob=0.0, seed=0):
     """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
-    fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask and slopes.
+    fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask, slopes, dropout
+    probability and seed.
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
     import torch
@@ -301,7 +305,8 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
                         lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), softmax_scale, causal,
                         window_left, window_right, FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16,
                         n_kv_heads=0 if Nk == N else Nk, S_kv=0 if S_kv == S else S_kv,
-                        alibi_ptr=0 if alibi_slopes is None else alibi_slopes.data_ptr(), strides=strides)
+                        alibi_ptr=0 if alibi_slopes is None else alibi_slopes.data_ptr(), strides=strides,
+                        dropout_prob=dropout_prob, seed=seed)
     need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
     workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), need

@@ -21,6 +21,9 @@ struct FaBwdArgs {
     int S, Sk;                              // queries, keys; query i sits at key position i + Sk - S
     int L, R;                               // key j visible to the query at position p iff p - L <= j <= p + R
     float scale;
+    unsigned drop_threshold;                // dropout: keep iff the key's byte >= threshold (p in units of 1/256); 0 = none
+    float drop_scale;                       // 256 / (256 - threshold)
+    unsigned seed_lo, seed_hi;
 };
 
 #endif

@@ -1,545 +1,12 @@
-// FlashAttention backward for gfx950 (MI355X): dQ, dK, dV from Q, K, V, O, dO and the logsumexp the forward
-// pass writes.  The reference has no backward pass (its L output is accepted and never written, reference
-// src/flash_forward.h:602,628-644); this is the consumer of the logsumexp this library emits.
-//
-//   P  = exp(scale * Q K^T - LSE)            (recomputed; masked pairs are 0)
-//   dV = P^T dO
-//   dP = dO V^T,   delta_i = sum_t dO_it O_it
-//   dS = P o (dP - delta)
-//   dQ = scale * dS K,   dK = scale * dS^T Q
-//
-// Two kernels: fa_bwd_dq (a workgroup owns 256 queries and walks the key tiles; it also writes delta and the
-// rescaled logsumexp for the second kernel) and fa_bwd_dkdv (a workgroup owns 256 keys of one K/V head and walks
-// the query tiles of the query heads that share it); no atomics, every output element has one writer, results
-// are the same bits from run to run.
-// Template flags: GENERAL = strides, any lengths (query i at key position i + Sk - S), grouped K/V heads;
-// the other instantiations assume contiguous [B,H,S,D] with S a multiple of 128 and keep their instruction
-// stream free of all that.  ALIBI (GENERAL only) subtracts slope[h] * |position - key| from the scaled score.
-// Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B
-// operands loaded once into registers, the walked tiles are A operands streamed through LDS by direct
-// global->LDS loads, and an accumulator tile is already laid out as the B operand of the next product.
-// A walked tile that is needed both row-wise (ds_read_b128) and transposed (ds_read_b64_tr_b16) sits in LDS
-// once, under a swizzle that is bank-conflict-free for both.
-#include "fa_fwd_kernel_impl.h"
-#include "fa_bwd_args.h"
-
-namespace {
-
-constexpr int kBwdWaves = 8;            // 8 waves x 32 owned rows = 256 rows per workgroup, two waves per SIMD
-constexpr int kBwdStages = 3;           // LDS ring: with three stages one barrier per tile is enough
-constexpr float kLog2e = 1.44269504088896340736f;
-
-// Takes the word by value on purpose: __builtin_bit_cast applied directly to an element of a vector
-// (`__builtin_bit_cast(float, v[e])`) reads element 0 whatever e is with this compiler.
-__device__ __forceinline__ float as_f32(uint32_t w) { return __builtin_bit_cast(float, w); }
-
-// One 16-byte-chunk swizzle that serves both read patterns of a walked tile, so that the tile sits in LDS once:
-// ds_read_b128 by 16 lanes on 16 consecutive rows and one logical chunk needs 16 different chunk positions
-// (a bijection of the row's low bits), ds_read_b64_tr_b16 by 32 lanes on 4 consecutive rows x 4 consecutive
-// chunks needs the 4 rows in 4 different 64-byte groups (the two high bits follow the row's low bits).
-// Invariant under row += 16, not under row += 8.
-template <int CPR> __device__ __forceinline__ int u_swz(int row)
-{
-    return CPR == 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
-}
-
-// per-lane LDS addresses of the two read patterns in the stage being read; everything else about a fragment
-// (which of the stage's tiles, which 32-row block, which 16-row slice) is an immediate offset of the read
-template <int D> struct TileReader {
-    static constexpr int CPR = D / 8, ROWB = D * 2, KS = D / 16, DB = D / 32;
-    uint32_t row_addr[KS];      // ds_read_b128: A operand rows = tile rows, k = 16 head-dim values of slice s
-    uint32_t tr_addr[DB][2];    // ds_read_b64_tr_b16: A operand rows = head dim (block db), k = 16 tile rows (two reads of 8)
-    __device__ __forceinline__ void init(int lane, uint32_t stage_base)
-    {
-        const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) row_addr[s] = stage_base + (uint32_t)(l32 * ROWB + (((2 * s + half) ^ u_swz<CPR>(l32)) << 4));
-        const int row0 = 4 * half + (l16 >> 2), dq = l32 >> 4, c4 = l16 & 3;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int hi = 0; hi < 2; ++hi) {
-                const int c = 4 * db + 2 * dq + (c4 >> 1), row = row0 + 8 * hi;
-                tr_addr[db][hi] = stage_base + (uint32_t)(row * ROWB + ((c ^ u_swz<CPR>(row)) << 4) + ((c4 & 1) << 3));
-            }
-    }
-    // move to another stage of the ring (delta in bytes, wave-uniform)
-    __device__ __forceinline__ void advance(int delta)
-    {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) row_addr[s] += delta;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) { tr_addr[db][0] += delta; tr_addr[db][1] += delta; }
-    }
-    // row-wise fragment: head-dim slice s, 32-row block b of the tile at byte `tile` of the stage
-    __device__ __forceinline__ u32x4 rows(int tile, int s, int b) const { return lds_read_b128(row_addr[s] + (uint32_t)(tile + b * 32 * ROWB)); }
-    // transposed fragment: 16-row slice t2, head-dim block db of the tile at byte `tile` of the stage
-    __device__ __forceinline__ u32x4 transposed(int tile, int t2, int db) const
-    {
-        const u32x2 lo = lds_read_tr(tr_addr[db][0] + (uint32_t)(tile + (16 * t2) * ROWB));
-        const u32x2 hi = lds_read_tr(tr_addr[db][1] + (uint32_t)(tile + (16 * t2) * ROWB));
-        return u32x4{lo[0], lo[1], hi[0], hi[1]};
-    }
-};
-
-// one 64-row tile global -> LDS: wave w issues instructions w, w+8, ...
-template <int D> struct TileLoader {
-    static constexpr int CPR = D / 8, ROWB = D * 2, TILEB = 64 * ROWB, IPW = TILEB / 1024 / kBwdWaves;
-    uint32_t g[IPW];
-    int wave, lane;
-    // row_bytes: distance between consecutive rows of the source in bytes
-    __device__ __forceinline__ void init(int wave_, int lane_, int row_bytes)
-    {
-        wave = wave_; lane = lane_;
-#pragma unroll
-        for (int i = 0; i < IPW; ++i) {
-            const int P = (i * kBwdWaves + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
-            g[i] = (uint32_t)(row * row_bytes + ((pos ^ u_swz<CPR>(row)) << 4));
-        }
-    }
-    __device__ __forceinline__ void load(const uint16_t *tile_src, uint32_t lds_tile) const
-    {
-#pragma unroll
-        for (int i = 0; i < IPW; ++i)
-            dma_16(reinterpret_cast<const char *>(tile_src), g[i], lds_tile + (i * kBwdWaves + wave) * 1024);
-    }
-    // a tile whose last rows lie past the end of the tensor: they are filled with copies of row `valid - 1`
-    __device__ __forceinline__ void load_ragged(const uint16_t *tile_src, uint32_t lds_tile, int valid, int row_bytes) const
-    {
-        // (the empty asm keeps the address arithmetic of this rare path inside its branch: hoisted out of the
-        // tile loop it would occupy registers for the whole kernel)
-        int ln = lane;
-        asm volatile("" : "+v"(ln));
-#pragma unroll
-        for (int i = 0; i < IPW; ++i) {
-            const int P = (i * kBwdWaves + wave) * 64 + ln, row = P / CPR, pos = P % CPR;
-            const int src_row = row < valid ? row : valid - 1;
-            dma_16(reinterpret_cast<const char *>(tile_src), (uint32_t)(src_row * row_bytes + ((pos ^ u_swz<CPR>(row)) << 4)),
-                   lds_tile + (i * kBwdWaves + wave) * 1024);
-        }
-    }
-};
-
-// 256 bytes (64 floats) global -> LDS in one wave instruction: lane l copies the float at src[index] to LDS
-// byte lds + 4*l
-__device__ __forceinline__ void dma_4(const float *src, int index, uint32_t lds)
-{
-    const uint64_t b = (uint64_t)src;
-    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
-    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
-    const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
-    const uint32_t voff = (uint32_t)index * 4u;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory");
-}
-
-__device__ __forceinline__ f32x16 zero16()
-{
-    f32x16 z;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
-    return z;
-}
-
-__device__ __forceinline__ const uint16_t *head_ptr(const uint16_t *p, const FaBwdTensor &t, int b, int h)
-{
-    return p + (long long)b * t.bs + (long long)h * t.hs;
-}
-__device__ __forceinline__ uint16_t *head_ptr(uint16_t *p, const FaBwdTensor &t, int b, int h)
-{
-    return p + (long long)b * t.bs + (long long)h * t.hs;
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// dQ: a workgroup owns 256 queries (lane = query), walks the key tiles of its visible range.
-// LDS stage: K (read row-wise for S^T = K Q^T and transposed for dQ^T += K^T dS^T), V (row-wise, dP^T = V dO^T).
-// ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI>
-__global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a)
-{
-    static_assert(!GENERAL || MASKED, "the general instantiations always carry the mask code (ragged tiles need it)");
-    static_assert(!ALIBI || GENERAL, "ALiBi is instantiated for the general layout only");
-    typedef Num<BF16> N;
-    typedef TileReader<D> Reader;
-    typedef TileLoader<D> Loader;
-    constexpr int KS = Reader::KS, DB = Reader::DB, TILEB = Loader::TILEB, STAGEB = 2 * TILEB, IPW = Loader::IPW;
-    extern __shared__ __attribute__((aligned(1024))) char smem[];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
-    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int S = a.S, Sk = GENERAL ? a.Sk : a.S, off = GENERAL ? a.Sk - a.S : 0;
-    const int n_qblocks = (S + 255) / 256;
-    // one head per XCD at a time, long blocks first: the workgroups that share a head's K and V share an L2
-    int bh, qblock;
-    fa_item_decode((long long)blockIdx.x, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
-    const int b = bh / a.H, h = bh - b * a.H, hk = GENERAL ? h / (a.H / a.Hk) : h;
-    const int q_rs = GENERAL ? a.q.rs : D, k_rs = GENERAL ? a.k.rs : D, v_rs = GENERAL ? a.v.rs : D;
-    const int o_rs = GENERAL ? a.o.rs : D, g_rs = GENERAL ? a.dO_.rs : D, dq_rs = GENERAL ? a.dq.rs : D;
-    const uint16_t *Qh, *Kh, *Vh, *Oh, *dOh;
-    uint16_t *dQh;
-    if (GENERAL) {
-        Qh = head_ptr(a.Q, a.q, b, h); Kh = head_ptr(a.K, a.k, b, hk); Vh = head_ptr(a.V, a.v, b, hk);
-        Oh = head_ptr(a.O, a.o, b, h); dOh = head_ptr(a.dO, a.dO_, b, h); dQh = head_ptr(a.dQ, a.dq, b, h);
-    } else {
-        const size_t head_off = (size_t)bh * S * D;
-        Qh = a.Q + head_off; Kh = a.K + head_off; Vh = a.V + head_off; Oh = a.O + head_off; dOh = a.dO + head_off;
-        dQh = a.dQ + head_off;
-    }
-    const int q0 = qblock * 256, qw = q0 + wave * 32;
-    const bool active = qw < S;                    // the last block may own fewer than 256 rows
-    const int my_q = active ? (GENERAL && qw + l32 >= S ? S - 1 : qw + l32) : (GENERAL ? 0 : l32);   // row to load
-    const bool row_ok = active && qw + l32 < S;
-    const int my_pos = qw + l32 + off;             // key position of this lane's query (masks, ALiBi)
-
-    u32x4 qf[KS], gf[KS];           // Q^T and dO^T as B operands: lane = (query, head-dim slice 8*half..+7 of each 16)
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        qf[s] = *reinterpret_cast<const u32x4 *>(Qh + (size_t)my_q * q_rs + 16 * s + 8 * half);
-        gf[s] = *reinterpret_cast<const u32x4 *>(dOh + (size_t)my_q * g_rs + 16 * s + 8 * half);
-    }
-    // logsumexp in exp2 units; a row that saw no key has -inf there and takes +inf here, which makes every P 0
-    const float lse_raw = a.lse[(size_t)bh * S + my_q];
-    float lse_l2 = (GENERAL && lse_raw == -INFINITY) ? INFINITY : lse_raw * kLog2e;
-    // delta_i = sum_t dO_it O_it: this lane holds half of row i of dO already; the other half is on lane ^ 32.
-    // Both are written out for fa_bwd_dkdv, which runs after this kernel.
-    float delta = 0.0f;
-    {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            const u32x4 o = *reinterpret_cast<const u32x4 *>(Oh + (size_t)my_q * o_rs + 16 * s + 8 * half);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const uint32_t ow = o[w], gw = gf[s][w];
-                delta += storage_to_f32<BF16>((uint16_t)(ow & 0xffffu)) * storage_to_f32<BF16>((uint16_t)(gw & 0xffffu));
-                delta += storage_to_f32<BF16>((uint16_t)(ow >> 16)) * storage_to_f32<BF16>((uint16_t)(gw >> 16));
-            }
-        }
-        delta += swap_halves(delta);
-        if (row_ok && half == 0) {
-            a.delta[(size_t)bh * S + my_q] = delta;
-            a.lse2[(size_t)bh * S + my_q] = lse_l2;
-        }
-    }
-    const float c = a.scale * kLog2e;
-    float slope_l2 = 0.0f;
-    if (ALIBI) slope_l2 = a.alibi[h] * kLog2e;
-
-    int t0, t1, my_lo = 1, my_hi = 0;
-    fa_tile_range(Sk, 64, a.L, a.R, q0 + off, S - q0 < 256 ? S - q0 : 256, &t0, &t1);
-    if (active) fa_tile_range(Sk, 64, a.L, a.R, qw + off, GENERAL && S - qw < 32 ? S - qw : 32, &my_lo, &my_hi);
-
-    Reader rd; rd.init(lane, lds0);
-    Loader ldk, ldv;
-    ldk.init(wave, lane, k_rs * 2);
-    if (GENERAL) ldv.init(wave, lane, v_rs * 2);
-    auto issue = [&](int tile, int stage) __attribute__((always_inline)) {
-        const uint32_t base = lds0 + stage * STAGEB;
-        if (GENERAL && (tile + 1) * 64 > Sk) {
-            ldk.load_ragged(Kh + (size_t)tile * 64 * k_rs, base, Sk - tile * 64, k_rs * 2);
-            ldv.load_ragged(Vh + (size_t)tile * 64 * v_rs, base + TILEB, Sk - tile * 64, v_rs * 2);
-        } else {
-            ldk.load(Kh + (size_t)tile * 64 * k_rs, base);
-            (GENERAL ? ldv : ldk).load(Vh + (size_t)tile * 64 * v_rs, base + TILEB);
-        }
-    };
-
-    f32x16 dq[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) dq[db] = zero16();
-
-    // 32 keys (block kb of the tile in the stage being read) against this wave's 32 queries
-    auto half_tile = [&](bool edge, int t, int kb) __attribute__((always_inline)) {
-        constexpr int k_tile = 0, v_tile = TILEB;
-        f32x16 sx = zero16(), dp = zero16();
-#pragma unroll
-        for (int s = 0; s < KS; ++s) sx = N::mfma(rd.rows(k_tile, s, kb), qf[s], sx);      // S^T = K Q^T
-#pragma unroll
-        for (int s = 0; s < KS; ++s) dp = N::mfma(rd.rows(v_tile, s, kb), gf[s], dp);      // dP^T = V dO^T
-        const int first = t * 64 + 32 * kb + 4 * half;                      // key of accumulator row 0 on this lane
-        if (MASKED && edge) {            // wave-uniform; a masked score becomes -inf and its P exactly 0
-            int hi = my_pos + a.R, lo = my_pos - a.L - first;                // visible: lo <= 8*(r/4) + r%4 <= hi
-            if (GENERAL && hi > Sk - 1) hi = Sk - 1;
-            hi -= first;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (8 * (r >> 2) + (r & 3) > hi || 8 * (r >> 2) + (r & 3) < lo) sx[r] = -INFINITY;
-        }
-        uint32_t ds[8];                                  // dS^T in B-operand order
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float v[2];
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int r = 2 * i + e;
-                float x = __builtin_fmaf(sx[r], c, -lse_l2);
-                if (ALIBI) x = __builtin_fmaf(-slope_l2, __builtin_fabsf((float)(first + 8 * (r >> 2) + (r & 3) - my_pos)), x);
-                const float p = __builtin_amdgcn_exp2f(x);
-                v[e] = p * (dp[r] - delta);
-            }
-            ds[i] = N::pack2(v[0], v[1]);
-        }
-#pragma unroll
-        for (int n = 0; n < 2 * DB; ++n) {                // dQ^T += K^T dS^T
-            const int h2 = n / DB, db = n % DB;
-            const u32x4 bfrag = {ds[4 * h2], ds[4 * h2 + 1], ds[4 * h2 + 2], ds[4 * h2 + 3]};
-            dq[db] = N::mfma(rd.transposed(k_tile, 2 * kb + h2, db), bfrag, dq[db]);
-        }
-    };
-
-    if (t0 <= t1) {
-        issue(t0, 0);
-        wait_vm<0>();
-        // the owner's operands have landed too: say so, or the compiler waits for them inside the loop, where
-        // its wait would also cover the asynchronous tile loads
-#pragma unroll
-        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]), "+v"(gf[s]));
-        asm volatile("" : "+v"(lse_l2), "+v"(delta), "+v"(slope_l2));
-        int stage = 0;
-        for (int t = t0; t <= t1; ++t) {
-            const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
-            if (t + 1 <= t1) { issue(t + 1, next); wait_vm<2 * IPW>(); }
-            else wait_vm<0>();
-            phase_barrier();                                    // tile t is in LDS for everyone; tile t-2's stage is free
-            if (my_lo <= t && t <= my_hi) {
-                const bool edge = MASKED && (fa_tile_class(64, a.L, a.R, qw + off, 32, t) == 1 || (GENERAL && (t + 1) * 64 > Sk));
-                half_tile(edge, t, 0);
-                half_tile(edge, t, 1);
-            }
-            rd.advance(next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB);
-            stage = next;
-        }
-    }
-    if (row_ok) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 w;
-                w[0] = N::pack2(dq[db][4 * g] * a.scale, dq[db][4 * g + 1] * a.scale);
-                w[1] = N::pack2(dq[db][4 * g + 2] * a.scale, dq[db][4 * g + 3] * a.scale);
-                *reinterpret_cast<u32x2 *>(dQh + (size_t)my_q * dq_rs + 32 * db + 8 * g + 4 * half) = w;
-            }
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// dK, dV: a workgroup owns 256 keys of one K/V head (lane = key), walks the query tiles that see them, for each
-// of the query heads that share the K/V head.
-// LDS stage: Q (row-wise for S = Q K^T, transposed for dK^T += Q^T dS), dO (row-wise for dP = dO V^T, transposed
-// for dV^T += dO^T P), 64 rescaled logsumexps, 64 deltas.
-// ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI>
-__global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
-{
-    typedef Num<BF16> N;
-    typedef TileReader<D> Reader;
-    typedef TileLoader<D> Loader;
-    constexpr int KS = Reader::KS, DB = Reader::DB, TILEB = Loader::TILEB, STAGEB = 2 * TILEB + 512, IPW = Loader::IPW;
-    extern __shared__ __attribute__((aligned(1024))) char smem[];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
-    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int S = a.S, Sk = GENERAL ? a.Sk : a.S, off = GENERAL ? a.Sk - a.S : 0;
-    const int G = GENERAL ? a.H / a.Hk : 1;
-    const int n_kblocks = (Sk + 255) / 256;
-    // one K/V head per XCD at a time; key block 0 is seen by the most queries and goes first
-    int bhk, kblock;
-    fa_item_decode((long long)blockIdx.x, a.B * a.Hk, n_kblocks, 0, &bhk, &kblock);
-    const int b = bhk / a.Hk, hk = bhk - b * a.Hk;
-    const int q_rs = GENERAL ? a.q.rs : D, g_rs = GENERAL ? a.dO_.rs : D, k_rs = GENERAL ? a.k.rs : D, v_rs = GENERAL ? a.v.rs : D;
-    const int dk_rs = GENERAL ? a.dk.rs : D, dv_rs = GENERAL ? a.dv.rs : D;
-    const uint16_t *Kh, *Vh;
-    uint16_t *dKh, *dVh;
-    if (GENERAL) {
-        Kh = head_ptr(a.K, a.k, b, hk); Vh = head_ptr(a.V, a.v, b, hk);
-        dKh = head_ptr(a.dK, a.dk, b, hk); dVh = head_ptr(a.dV, a.dv, b, hk);
-    } else {
-        const size_t head_off = (size_t)bhk * S * D;
-        Kh = a.K + head_off; Vh = a.V + head_off; dKh = a.dK + head_off; dVh = a.dV + head_off;
-    }
-    const int k0 = kblock * 256, kw = k0 + wave * 32;
-    const bool active = kw < Sk;
-    const int my_k = kw + l32;                     // this lane's key (masks, ALiBi)
-    const int my_kc = active ? (GENERAL && my_k >= Sk ? Sk - 1 : my_k) : (GENERAL ? 0 : l32);     // row to load
-    const bool row_ok = active && my_k < Sk;
-
-    u32x4 kf[KS], vf[KS];           // K^T and V^T as B operands: lane = (key, head-dim slice)
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        kf[s] = *reinterpret_cast<const u32x4 *>(Kh + (size_t)my_kc * k_rs + 16 * s + 8 * half);
-        vf[s] = *reinterpret_cast<const u32x4 *>(Vh + (size_t)my_kc * v_rs + 16 * s + 8 * half);
-    }
-    const float c = a.scale * kLog2e;
-
-    // the query tiles that see these keys: the query at index i (position i + off) sees key j iff
-    // j - R - off <= i <= j + L - off: the forward bounds with the two sides exchanged and shifted
-    const int Lq = a.R + off, Rq = a.L - off;
-    int t0, t1, my_lo = 1, my_hi = 0;
-    fa_tile_range(S, 64, Lq, Rq, k0, Sk - k0 < 256 ? Sk - k0 : 256, &t0, &t1);
-    if (active) fa_tile_range(S, 64, Lq, Rq, kw, GENERAL && Sk - kw < 32 ? Sk - kw : 32, &my_lo, &my_hi);
-
-    Reader rd; rd.init(lane, lds0);
-    uint32_t stat_addr = lds0 + 2 * TILEB + 16 * half;       // this lane's logsumexp / delta words in the stage being read
-    Loader ldq, ldg;
-    ldq.init(wave, lane, q_rs * 2);
-    if (GENERAL) ldg.init(wave, lane, g_rs * 2);
-    // g: query head inside the group of this K/V head
-    auto issue = [&](int g, int tile, int stage) __attribute__((always_inline)) {
-        const uint32_t base = lds0 + stage * STAGEB;
-        const int h = hk * G + g;
-        const uint16_t *Qh, *dOh;
-        if (GENERAL) { Qh = head_ptr(a.Q, a.q, b, h); dOh = head_ptr(a.dO, a.dO_, b, h); }
-        else { Qh = a.Q + (size_t)bhk * S * D; dOh = a.dO + (size_t)bhk * S * D; }
-        const float *lse_h = a.lse2 + ((size_t)b * a.H + h) * S, *delta_h = a.delta + ((size_t)b * a.H + h) * S;
-        if (GENERAL && (tile + 1) * 64 > S) {
-            const int valid = S - tile * 64;
-            ldq.load_ragged(Qh + (size_t)tile * 64 * q_rs, base, valid, q_rs * 2);
-            ldg.load_ragged(dOh + (size_t)tile * 64 * g_rs, base + TILEB, valid, g_rs * 2);
-            int ln = lane;
-            asm volatile("" : "+v"(ln));
-            if (wave == 0) dma_4(lse_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB);
-            if (wave == 1) dma_4(delta_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB + 256);
-        } else {
-            ldq.load(Qh + (size_t)tile * 64 * q_rs, base);
-            (GENERAL ? ldg : ldq).load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
-            if (wave == 0) dma_4(lse_h + tile * 64, lane, base + 2 * TILEB);
-            if (wave == 1) dma_4(delta_h + tile * 64, lane, base + 2 * TILEB + 256);
-        }
-    };
-    f32x16 dk[DB], dv[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) { dk[db] = zero16(); dv[db] = zero16(); }
-
-    // 32 queries (block qb of the tile in the stage being read) against this wave's 32 keys
-    auto half_tile = [&](bool edge, float slope_l2, int t, int qb) __attribute__((always_inline)) {
-        constexpr int q_tile = 0, g_tile = TILEB;
-        f32x16 sx = zero16();            // rows = queries, column (lane) = key
-#pragma unroll
-        for (int s = 0; s < KS; ++s) sx = N::mfma(rd.rows(q_tile, s, qb), kf[s], sx);      // S = Q K^T
-        const int first = t * 64 + 32 * qb + 4 * half;                      // query of accumulator row 0 on this lane
-        if (MASKED && edge) {            // wave-uniform; a masked score becomes -inf and its P exactly 0
-            int hi = my_k + Rq, lo = my_k - Lq - first;                      // visible: lo <= 8*(r/4) + r%4 <= hi
-            if (GENERAL && hi > S - 1) hi = S - 1;
-            hi -= first;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (8 * (r >> 2) + (r & 3) > hi || 8 * (r >> 2) + (r & 3) < lo) sx[r] = -INFINITY;
-        }
-        // accumulator row r is query 32*qb + 8*(r/4) + 4*half + r%4 of the tile
-        uint32_t pp[8];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const u32x4 lraw = lds_read_b128(stat_addr + (uint32_t)(32 * qb + 8 * g) * 4u);
-            float p[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int r = 4 * g + e;
-                float x = __builtin_fmaf(sx[r], c, -as_f32(lraw[e]));
-                if (ALIBI) x = __builtin_fmaf(-slope_l2, __builtin_fabsf((float)(first + 8 * g + e + off - my_k)), x);
-                p[e] = __builtin_amdgcn_exp2f(x);
-                sx[r] = p[e];                    // keep P in fp32 for dS
-            }
-            pp[2 * g] = N::pack2(p[0], p[1]);
-            pp[2 * g + 1] = N::pack2(p[2], p[3]);
-        }
-#pragma unroll
-        for (int n = 0; n < 2 * DB; ++n) {                // dV^T += dO^T P
-            const int h2 = n / DB, db = n % DB;
-            const u32x4 bfrag = {pp[4 * h2], pp[4 * h2 + 1], pp[4 * h2 + 2], pp[4 * h2 + 3]};
-            dv[db] = N::mfma(rd.transposed(g_tile, 2 * qb + h2, db), bfrag, dv[db]);
-        }
-        f32x16 dp = zero16();
-#pragma unroll
-        for (int s = 0; s < KS; ++s) dp = N::mfma(rd.rows(g_tile, s, qb), vf[s], dp);      // dP = dO V^T
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const u32x4 draw = lds_read_b128(stat_addr + 256u + (uint32_t)(32 * qb + 8 * g) * 4u);
-            float v[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = sx[4 * g + e] * (dp[4 * g + e] - as_f32(draw[e]));
-            pp[2 * g] = N::pack2(v[0], v[1]);     // now dS, same operand order
-            pp[2 * g + 1] = N::pack2(v[2], v[3]);
-        }
-#pragma unroll
-        for (int n = 0; n < 2 * DB; ++n) {                // dK^T += Q^T dS
-            const int h2 = n / DB, db = n % DB;
-            const u32x4 bfrag = {pp[4 * h2], pp[4 * h2 + 1], pp[4 * h2 + 2], pp[4 * h2 + 3]};
-            dk[db] = N::mfma(rd.transposed(q_tile, 2 * qb + h2, db), bfrag, dk[db]);
-        }
-    };
-
-    if (t0 <= t1) {
-        // from the last query tile down to the diagonal: every workgroup of a head then starts on the same tile
-        // and the ones that run together keep reading the same tiles out of L2; then the next head of the group
-        issue(0, t1, 0);
-        wait_vm<0>();
-#pragma unroll
-        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
-        int stage = 0;
-        for (int g = 0; g < G; ++g) {
-            float slope_l2 = 0.0f;
-            if (ALIBI) slope_l2 = a.alibi[hk * G + g] * kLog2e;
-            for (int t = t1; t >= t0; --t) {
-                const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
-                const bool more = t - 1 >= t0 || g + 1 < G;
-                if (more) {
-                    if (t - 1 >= t0) issue(g, t - 1, next); else issue(g + 1, t1, next);
-                    if (wave < 2) wait_vm<2 * IPW + 1>(); else wait_vm<2 * IPW>();     // waves 0 and 1 also fetch lse / delta
-                } else wait_vm<0>();
-                phase_barrier();
-                if (my_lo <= t && t <= my_hi) {
-                    const bool edge = MASKED && (fa_tile_class(64, Lq, Rq, kw, 32, t) == 1 || (GENERAL && (t + 1) * 64 > S));
-                    half_tile(edge, slope_l2, t, 0);
-                    half_tile(edge, slope_l2, t, 1);
-                }
-                rd.advance(next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB);
-                stat_addr += next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB;
-                stage = next;
-            }
-        }
-    }
-    if (row_ok) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 wk, wv;
-                wk[0] = N::pack2(dk[db][4 * g] * a.scale, dk[db][4 * g + 1] * a.scale);
-                wk[1] = N::pack2(dk[db][4 * g + 2] * a.scale, dk[db][4 * g + 3] * a.scale);
-                wv[0] = N::pack2(dv[db][4 * g], dv[db][4 * g + 1]);
-                wv[1] = N::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
-                *reinterpret_cast<u32x2 *>(dKh + (size_t)my_kc * dk_rs + 32 * db + 8 * g + 4 * half) = wk;
-                *reinterpret_cast<u32x2 *>(dVh + (size_t)my_kc * dv_rs + 32 * db + 8 * g + 4 * half) = wv;
-            }
-    }
-}
-
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI>
-hipError_t launch_bwd(const FaBwdArgs &a, hipStream_t stream)
-{
-    constexpr int TILEB = 64 * D * 2;
-    const unsigned grid_q = (unsigned)((long long)a.B * a.H * ((a.S + 255) / 256));
-    const unsigned grid_k = (unsigned)((long long)a.B * a.Hk * ((a.Sk + 255) / 256));
-    const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512);
-    auto kq = fa_bwd_dq<BF16, D, MASKED, GENERAL, ALIBI>;
-    auto kkv = fa_bwd_dkdv<BF16, D, MASKED, GENERAL, ALIBI>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kq), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kq, dim3(grid_q), dim3(kBwdWaves * 64), smem_dq, stream, a);
-    hipLaunchKernelGGL(kkv, dim3(grid_k), dim3(kBwdWaves * 64), smem_dkdv, stream, a);
-    return hipGetLastError();
-}
-
-}  // namespace
+// Backward kernels without dropout: the instantiations for the reference's layout and the general ones.
+#include "fa_bwd_kernel_impl.h"
 
 // general: strides, any lengths, grouped K/V heads (always with the mask code); alibi needs general
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, hipStream_t stream)
 {
 #define FA_BWD_CASE(BF, DD, MK, GN, AL) \
     if (bf16 == BF && D == DD && masked == MK && general == GN && alibi == AL) \
-        return launch_bwd<BF != 0, DD, MK != 0, GN != 0, AL != 0>(a, stream);
+        return launch_bwd<BF != 0, DD, MK != 0, GN != 0, AL != 0, false>(a, stream);
     FA_BWD_CASE(0, 64, 0, 0, 0) FA_BWD_CASE(0, 64, 1, 0, 0) FA_BWD_CASE(0, 128, 0, 0, 0) FA_BWD_CASE(0, 128, 1, 0, 0)
     FA_BWD_CASE(1, 64, 0, 0, 0) FA_BWD_CASE(1, 64, 1, 0, 0) FA_BWD_CASE(1, 128, 0, 0, 0) FA_BWD_CASE(1, 128, 1, 0, 0)
     FA_BWD_CASE(0, 64, 1, 1, 0) FA_BWD_CASE(0, 128, 1, 1, 0) FA_BWD_CASE(1, 64, 1, 1, 0) FA_BWD_CASE(1, 128, 1, 1, 0)

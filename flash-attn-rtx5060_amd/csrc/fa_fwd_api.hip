@@ -27,6 +27,7 @@ hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int
                                      hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, hipStream_t stream);
+hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, hipStream_t stream);
 hipError_t fa_work_queue_base(unsigned **base);
 int fa_work_queue_slots();
 
@@ -450,6 +451,7 @@ int fa_bwd_validate(const fa_bwd_params *p)
     if (p->dtype != FA_DTYPE_F16 && p->dtype != FA_DTYPE_BF16) return FA_ERR_DTYPE;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
+    if (!(p->dropout_prob >= 0.0f) || !(p->dropout_prob < 1.0f)) return FA_ERR_UNSUPPORTED;
     const long long s_kv = p->S_kv > 0 ? p->S_kv : p->S;
     if ((long long)p->B * p->N * ((p->S + 255) / 256) > 0x7fffffffLL || (long long)p->B * p->N * ((s_kv + 255) / 256) > 0x7fffffffLL ||
         (long long)p->S + s_kv > 0x3fffffffLL) return FA_ERR_TOO_LARGE;
@@ -515,9 +517,15 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     const int far = a.S + a.Sk;
     fa_mask_bounds(far, p->is_causal, p->window_size_left, p->window_size_right, &a.L, &a.R);
     a.scale = p->softmax_scale;
+    a.drop_threshold = (unsigned)fa_dropout_threshold(p->dropout_prob);
+    a.drop_scale = 256.0f / (256.0f - (float)a.drop_threshold);
+    a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
+    a.seed_hi = (unsigned)(p->seed >> 32);
     const int masked = (general || a.L < far || a.R < far) ? 1 : 0;
-    hipError_t e = fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general ? 1 : 0, a.alibi != nullptr ? 1 : 0,
-                                      static_cast<hipStream_t>(stream));
+    hipError_t e = a.drop_threshold != 0
+        ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, static_cast<hipStream_t>(stream))
+        : fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general ? 1 : 0, a.alibi != nullptr ? 1 : 0,
+                             static_cast<hipStream_t>(stream));
     return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
 }
 

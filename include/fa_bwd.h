@@ -8,8 +8,8 @@
  *
  * Layouts as in fa_fwd(): fp16 or bf16, d 64 or 128, any S >= 1, contiguous [B,N,S,d] or element strides with a
  * contiguous last dimension, K/V with n_kv_heads heads (dK and dV are summed over the query heads of a group) and
- * S_kv keys (query i sits at key position i + S_kv - S), causal and one- or two-sided window masks, ALiBi.
- * Not in the parameter block, hence not supported: dropout, key splits.
+ * S_kv keys (query i sits at key position i + S_kv - S), causal and one- or two-sided window masks, ALiBi,
+ * dropout (the forward's decisions are replayed from its seed, nothing is stored).  Key splits do not apply.
  */
 #ifndef FA_BWD_H
 #define FA_BWD_H
@@ -44,6 +44,8 @@ typedef struct fa_bwd_params {
     long long dq_strides[3];
     long long dk_strides[3];
     long long dv_strides[3];
+    float dropout_prob;       /* the forward's; 0 = none.  The keep decisions are replayed from (seed, head, query, key) */
+    unsigned long long seed;  /* the forward's                                                                  */
 } fa_bwd_params;
 
 int fa_bwd_validate(const fa_bwd_params *p);

@@ -69,12 +69,12 @@ def test_backward_struct_layout_and_status_codes(fa):
         with open(src, "w") as f:
             f.write('#include <stdio.h>\n#include <stddef.h>\n#include "fa_bwd.h"\n'
                     'int main(void){printf("%zu %zu %zu\\n", sizeof(fa_bwd_params), offsetof(fa_bwd_params, softmax_scale),'
-                    ' offsetof(fa_bwd_params, dv_strides));return 0;}\n')
+                    ' offsetof(fa_bwd_params, seed));return 0;}\n')
         exe = os.path.join(tmp, "layout")
         subprocess.run(["gcc", "-I", os.path.join(REPO, "include"), src, "-o", exe], check=True)
         size, off_scale, off_ws = (int(x) for x in subprocess.run([exe], check=True, stdout=subprocess.PIPE, text=True).stdout.split())
     assert size == ctypes.sizeof(fa.FaBwdParams)
-    assert off_scale == fa.FaBwdParams.softmax_scale.offset and off_ws == fa.FaBwdParams.dv_strides.offset
+    assert off_scale == fa.FaBwdParams.softmax_scale.offset and off_ws == fa.FaBwdParams.seed.offset
 
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128, q_ptr=0x1000, k_ptr=0x2000, v_ptr=0x3000, o_ptr=0x4000, do_ptr=0x5000,
@@ -93,6 +93,7 @@ def test_backward_struct_layout_and_status_codes(fa):
     assert status(d=96) == fa.FA_ERR_HEAD_DIM
     assert status(S=1000) == fa.FA_OK and status(S_kv=-1) == fa.FA_ERR_BAD_SHAPE
     assert status(n_kv_heads=3) == fa.FA_ERR_LAYOUT and status(n_kv_heads=2) == fa.FA_OK
+    assert status(dropout_prob=1.0) == fa.FA_ERR_UNSUPPORTED and status(dropout_prob=0.3) == fa.FA_OK
     assert status(strides=dict(dk=(8, 8, 100))) == fa.FA_ERR_LAYOUT and status(strides=dict(q=(4 * 1024 * 256, 256, 4 * 256))) == fa.FA_OK
     assert status(dtype=7) == fa.FA_ERR_DTYPE
     assert status(softmax_scale=0.0) == fa.FA_ERR_SCALE and status(softmax_scale=float("nan")) == fa.FA_ERR_SCALE

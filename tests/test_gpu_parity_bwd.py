@@ -97,7 +97,7 @@ def test_backward_refuses_what_it_does_not_cover(fa):
     p = params(); p.dK = 0
     assert L.fa_bwd(ctypes.byref(p), None) == fa.FA_ERR_NULL_POINTER
 
-def oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes):
+def oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes, dropout=(0, 0)):
     """q, do [B,H,S,D], k, v [B,Hk,Skv,D] (storage bits) -> fp64 dq [B,H,S,D], dk, dv [B,Hk,Skv,D].
     The oracle differentiates square problems with one K/V head per query head.  Grouped heads: repeat K and V
     and sum their gradients over the group.  S < Skv: the queries are the last S rows of the square Skv problem
@@ -110,7 +110,7 @@ def oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes):
     qpad = np.zeros((B, H, Skv, D), dtype=np.uint16)
     dopad = np.zeros((B, H, Skv, D), dtype=np.uint16)
     qpad[:, :, off:], dopad[:, :, off:] = q, do
-    dq, dk, dv = oracle.bwd_f64(qpad, kf, vf, dopad, dtype, None, causal, wl, wr, slopes)
+    dq, dk, dv = oracle.bwd_f64(qpad, kf, vf, dopad, dtype, None, causal, wl, wr, slopes, dropout=dropout)
     return dq[:, :, off:], dk.reshape(B, Hk, rep, Skv, D).sum(axis=2), dv.reshape(B, Hk, rep, Skv, D).sum(axis=2)
 
 
@@ -171,3 +171,43 @@ def test_queries_without_any_key_get_zero_gradients(fa):
         err = grad_errors(got.float().cpu().numpy(), want.cpu().numpy())
         print("blind rows", name, err, flush=True)
         check(err, 0, name)
+
+
+DROPOUT = [
+    # B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd, p, seed
+    (1, 2, 2, 256, 256, 64, 0, False, -1, -1, False, False, 0.1, 48),
+    (2, 2, 2, 384, 384, 128, 0, True, -1, -1, False, False, 0.1, 48),
+    (1, 4, 2, 333, 333, 128, 0, True, -1, -1, False, True, 0.25, 0x123456789ABCDEF),     # grouped heads, ragged, [B,S,H,D]
+    (1, 2, 2, 200, 456, 128, 1, True, -1, -1, False, False, 0.5, 7),                     # more keys than queries, bf16
+    (1, 2, 1, 190, 190, 64, 0, False, 50, 30, True, False, 0.2, 8),                      # ALiBi, window, one K/V head
+    (1, 3, 3, 640, 640, 128, 0, True, 100, -1, True, False, 0.9, 9),                     # almost everything dropped
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,Skv,D,dtype,causal,wl,wr,alibi,bshd,p,seed", DROPOUT)
+def test_dropout_gradients_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd, p, seed):
+    """The backward pass replays the forward's keep decisions from (seed, head, query position, key); the oracle
+    does the same on the CPU.  Kept probabilities are multiplied by 1/(1-p), and so is every rounding error."""
+    import torch
+    thr = fa.lib().fa_dropout_threshold(p)
+    q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=800 + S)
+    do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=801 + S)
+    _, k, v = make_inputs(fa, (B, Hk, Skv, D), dtype, seed=802 + Skv)
+    slopes = np.power(2.0, -8.0 / H * (np.arange(H) + 1)).astype(np.float32) if alibi else None
+    dq_ref, dk_ref, dv_ref = oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes, dropout=(thr, seed))
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    if bshd:
+        tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
+    ts = None if slopes is None else torch.from_numpy(slopes).cuda()
+    kw = dict(causal=causal, window_left=wl, window_right=wr, alibi_slopes=ts, dropout_prob=p, seed=seed)
+    o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
+    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
+    dq2, dk2, dv2 = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
+    torch.cuda.synchronize()
+    grow = 256.0 / (256 - thr)
+    rel, mx = (1e-3, 2e-3) if dtype == 0 else (8e-3, 1.6e-2)
+    for name, got, again, want in (("dQ", dq, dq2, dq_ref), ("dK", dk, dk2, dk_ref), ("dV", dv, dv2, dv_ref)):
+        err = grad_errors(oracle.to_f32(from_torch(got.contiguous()), dtype), want)
+        print((B, H, Hk, S, Skv, D), dtype, causal, wl, wr, alibi, bshd, p, name, err, flush=True)
+        assert err["nonfinite"] == 0 and err["rel_l2"] <= rel * grow and err["max_abs"] <= mx * grow * max(1.0, err["max_ref"]), (name, err)
+        assert torch.equal(got.view(torch.int16), again.view(torch.int16))        # no atomics: the same bits every time
