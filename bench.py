@@ -116,11 +116,12 @@ def backward_bench(args):
     q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed, sigma, frac, mult)
     do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed + 1000)
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
-    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl)
+    kw = dict(causal=causal, window_left=wl, dropout_prob=args.dropout, seed=48)
+    o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
     grads = [None]
 
     def step():
-        grads[0] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl)
+        grads[0] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -143,7 +144,12 @@ def backward_bench(args):
     if wl >= 0:
         vis &= i[:, None] - i[None, :] <= wl
     sc = (qf @ kf.T) * float(np.float32(1.0 / np.sqrt(D)))
-    (torch.softmax(sc.masked_fill(~vis, float("-inf")), dim=-1) @ vf).backward(tdo[-1, -1].float())
+    pm = torch.softmax(sc.masked_fill(~vis, float("-inf")), dim=-1)
+    if args.dropout > 0:
+        from parity_util import numpy_keep_mask
+        thr = fa.lib().fa_dropout_threshold(args.dropout)
+        pm = pm * torch.from_numpy(numpy_keep_mask(48, B * H - 1, S, thr).astype(np.float32) * (256.0 / (256 - thr))).cuda()
+    (pm @ vf).backward(tdo[-1, -1].float())
     err = {}
     for name, got, want in zip(("dQ", "dK", "dV"), grads[0], (qf.grad, kf.grad, vf.grad)):
         d = got[-1, -1].float() - want
@@ -154,7 +160,8 @@ def backward_bench(args):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
         "config": {"workload": f"{args.workload} backward: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D}"
-                               f"{' causal' if causal else ''}{f' window_left {wl}' if wl >= 0 else ''}",
+                               f"{' causal' if causal else ''}{f' window_left {wl}' if wl >= 0 else ''}"
+                               f"{f' dropout {args.dropout}' if args.dropout > 0 else ''}",
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4), "traffic": None,
