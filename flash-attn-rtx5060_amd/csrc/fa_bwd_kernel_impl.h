@@ -296,7 +296,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     };
 
     if (t0 <= t1) {
+        // Tiles are fetched two ahead: tile t+2 is issued at the end of iteration t, into the stage tile t-1 was
+        // read from (free for everyone since this iteration's barrier).  A wait for "everything in flight" in the
+        // middle of an iteration -- the compiler's own, around a register it spilled -- then only meets loads
+        // that were issued a whole iteration earlier.
         issue(t0, 0);
+        if (t0 + 1 <= t1) issue(t0 + 1, 1);
         wait_vm<0>();
         // the owner's operands have landed too: say so, or the compiler waits for them inside the loop, where
         // its wait would also cover the asynchronous tile loads
@@ -306,14 +311,15 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
         int stage = 0;
         for (int t = t0; t <= t1; ++t) {
             const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
-            if (t + 1 <= t1) { issue(t + 1, next); wait_vm<2 * IPW>(); }
+            if (t + 1 <= t1) wait_vm<2 * IPW>();                // tile t has landed, tile t+1 may still be in flight
             else wait_vm<0>();
-            phase_barrier();                                    // tile t is in LDS for everyone; tile t-2's stage is free
+            phase_barrier();                                    // tile t is in LDS for everyone; tile t-1's stage is free
             if (my_lo <= t && t <= my_hi) {
                 const bool edge = MASKED && (fa_tile_class(64, a.L, a.R, qw + off, 32, t) == 1 || (GENERAL && (t + 1) * 64 > Sk));
                 half_tile(edge, t, 0);
                 half_tile(edge, t, 1);
             }
+            if (t + 2 <= t1) issue(t + 2, next == kBwdStages - 1 ? 0 : next + 1);
             rd.advance(next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB);
             stage = next;
         }
@@ -511,7 +517,14 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     if (t0 <= t1) {
         // from the last query tile down to the diagonal: every workgroup of a head then starts on the same tile
         // and the ones that run together keep reading the same tiles out of L2; then the next head of the group
-        issue(0, t1, 0);
+        // (head, tile) pairs are fetched two ahead, as in fa_bwd_dq
+        int ig = 0, it = t1;                                    // the next pair to fetch
+        auto issue_next = [&](int stage) __attribute__((always_inline)) {
+            issue(ig, it, stage);
+            if (--it < t0) { it = t1; ++ig; }
+        };
+        issue_next(0);
+        if (ig < G) issue_next(1);
         wait_vm<0>();
 #pragma unroll
         for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
@@ -522,8 +535,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             for (int t = t1; t >= t0; --t) {
                 const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
                 const bool more = t - 1 >= t0 || g + 1 < G;
-                if (more) {
-                    if (t - 1 >= t0) issue(g, t - 1, next); else issue(g + 1, t1, next);
+                if (more) {                                     // this pair has landed, the next may still be in flight
                     if (wave < 2) wait_vm<2 * IPW + 1>(); else wait_vm<2 * IPW>();     // waves 0 and 1 also fetch lse / delta
                 } else wait_vm<0>();
                 phase_barrier();
@@ -533,6 +545,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
                     half_tile(edge, slope_l2, bhq, t, 0);
                     half_tile(edge, slope_l2, bhq, t, 1);
                 }
+                if (ig < G) issue_next(next == kBwdStages - 1 ? 0 : next + 1);
                 rd.advance(next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB);
                 stat_addr += next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB;
                 stage = next;
