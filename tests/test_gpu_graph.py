@@ -1,0 +1,42 @@
+"""The library under HIP graph capture: fa_fwd (work-queue schedule, whose per-XCD counters every launch leaves
+zeroed) and fa_bwd recorded once with torch.cuda.CUDAGraph and replayed on new inputs, each replay compared with
+an eager call.  Neither entry point allocates, synchronises or records a memset, so capture needs nothing special;
+the first (eager) call resolves the counters' device address, which is not a stream operation."""
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,sched", [((2, 8, 1024, 128), 3), ((1, 4, 256, 64), 1), ((4, 16, 2048, 64), 0)])
+def test_forward_and_backward_replayed_from_a_graph(fa, shape, sched):
+    import torch
+    B, H, S, D = shape
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v, do = (torch.randn(shape, device="cuda", generator=g).half() for _ in range(4))
+    o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+
+    def run(out, out_lse):
+        fa.flash_attention_forward(q, k, v, causal=True, out=out, lse=out_lse, sched=sched)
+        return fa.flash_attention_backward(q, k, v, out, out_lse, do, causal=True)
+
+    run(o, lse)                                     # eager warm-up: loads the kernels, resolves the work-queue address
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            grads = run(o, lse)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        for t in (q, k, v, do):                     # new contents in the captured tensors
+            t.copy_(torch.randn(shape, device="cuda", generator=g).half())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (o, lse, *grads)]
+        o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
+        want = [o2, lse2, *run(o2, lse2)]
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a.view(torch.int32 if a.dtype == torch.float32 else torch.int16),
+                               b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)), (replay, shape, sched)
