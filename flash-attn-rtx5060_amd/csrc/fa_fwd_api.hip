@@ -40,6 +40,7 @@ constexpr int kComputeUnits = 256;      // MI355X; the persistent grid is sized 
 // items and wins when there are too few of the large ones to fill and balance the chip.
 int waves_for(int B, int N, int S)
 {
+    if (S < 256) return 4;              // (few queries per head, e.g. decoding: a 256-row block would be mostly empty)
     const long long big_items = (long long)B * N * ((S + 255) / 256);
     return big_items >= 2LL * kComputeUnits ? 8 : 4;
 }
