@@ -316,6 +316,38 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     return dq, dk, dv
 
 
+_autograd_function = None
+
+
+def flash_attention(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1, alibi_slopes=None,
+                    dropout_prob=0.0, seed=0):
+    """Differentiable attention for PyTorch callers: fa_fwd in the forward pass, fa_bwd in the backward pass
+    (which replays the dropout decisions from ``seed``; nothing but O and the logsumexp is saved).  Shapes and
+    layouts as in flash_attention_forward.  Plumbing only: both passes are the library's kernels."""
+    global _autograd_function
+    import torch
+    if _autograd_function is None:
+        class _FlashAttention(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, q, k, v, opts):
+                o, lse = flash_attention_forward(q, k, v, **opts)
+                ctx.save_for_backward(q, k, v, o, lse)
+                ctx.opts = opts
+                return o
+
+            @staticmethod
+            def backward(ctx, do):
+                q, k, v, o, lse = ctx.saved_tensors
+                if do.stride(3) != 1:
+                    do = do.contiguous()
+                dq, dk, dv = flash_attention_backward(q, k, v, o, lse, do, **ctx.opts)
+                return dq, dk, dv, None
+        _autograd_function = _FlashAttention
+    opts = dict(softmax_scale=softmax_scale, causal=causal, window_left=window_left, window_right=window_right,
+                alibi_slopes=alibi_slopes, dropout_prob=dropout_prob, seed=seed)
+    return _autograd_function.apply(q, k, v, opts)
+
+
 def run_flash_attention(B, N, S, d, Q, K, V, O, L=None, M=None, Is_dropout=False, Is_causal=False, Is_local=False,
                         Has_alibi=False, window_size=0, alibi_slopes=None, dropout_prob=0.0, states=None):
     """The reference's entry point with its argument order (flash_forward.h:593-612); Q..L are torch

@@ -264,3 +264,26 @@ def test_small_and_odd_shapes_against_torch_autograd_f64(fa, B, H, Hk, S, Skv, D
         err = grad_errors(got.float().cpu().numpy(), want)
         print((B, H, Hk, S, Skv, D), dtype, causal, wl, wr, name, err, flush=True)
         check(err, dtype, name)
+
+
+def test_autograd_wrapper_trains_like_torch_attention(fa):
+    """fa.flash_attention under torch autograd: [B,S,H,D] storage, grouped K/V heads, a loss that is not a plain
+    sum, compared with torch's scaled_dot_product_attention differentiated in fp32."""
+    import torch
+    B, S, H, Hk, D = 2, 512, 8, 2, 128
+    g = torch.Generator(device="cuda").manual_seed(21)
+    base = [torch.randn((B, S, n, D), device="cuda", generator=g).half() for n in (H, Hk, Hk)]
+    w = torch.randn((B, H, S, D), device="cuda", generator=g).half()
+    q, k, v = (t.transpose(1, 2).detach().requires_grad_(True) for t in base)
+    out = fa.flash_attention(q, k, v, causal=True)
+    ((out.float() * w.float()).sum() + 0.5 * (out.float() ** 2).sum()).backward()
+    qf, kf, vf = (t.transpose(1, 2).detach().float().requires_grad_(True) for t in base)
+    ref = torch.nn.functional.scaled_dot_product_attention(qf, kf.repeat_interleave(H // Hk, 1), vf.repeat_interleave(H // Hk, 1), is_causal=True)
+    ((ref * w.float()).sum() + 0.5 * (ref ** 2).sum()).backward()
+    torch.cuda.synchronize()
+    assert float((out.detach().float() - ref.detach()).abs().max()) <= 2e-3
+    for name, got, want in (("dQ", q.grad, qf.grad), ("dK", k.grad, kf.grad), ("dV", v.grad, vf.grad)):
+        err = grad_errors(got.float().cpu().numpy(), want.cpu().numpy())
+        print("autograd wrapper", name, err, flush=True)
+        # the loss gradient dO = w + out is itself rounded to fp16 on the way into fa_bwd
+        assert err["nonfinite"] == 0 and err["rel_l2"] <= 2e-3 and err["max_abs"] <= 4e-3 * max(1.0, err["max_ref"]), (name, err)
