@@ -261,7 +261,8 @@ def main():
         "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None if (args.alibi or args.dropout) else MEASURED_HBM_BYTES.get(args.workload),
-                     "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
+                     "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_median": round(float(np.median(kernel_ms)), 5),
+                     "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
     }
 
     drop = (fa.lib().fa_dropout_threshold(args.dropout), 48)
