@@ -23,6 +23,8 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 # script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
 # worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 424.1 MB read + 137.0 MB written.
 MEASURED_HBM_BYTES = {"c3": 561.1e6}
+# the same for the two backward kernels together on c3's shape: 1756.4 MB read + 414.9 MB written
+MEASURED_BWD_HBM_BYTES = {"c3": 2171.3e6}
 
 WORKLOADS = {
     # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
@@ -164,7 +166,8 @@ def backward_bench(args):
                                f"{f' dropout {args.dropout}' if args.dropout > 0 else ''}",
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4),
+                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 else None,
                      "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_dq + fa_bwd_dkdv"},
         "parity_vs_torch_fp32_one_head": err}))
 
