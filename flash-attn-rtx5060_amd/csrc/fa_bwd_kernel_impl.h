@@ -15,9 +15,11 @@
 // Template flags: GENERAL = strides, any lengths (query i at key position i + Sk - S), grouped K/V heads;
 // the other instantiations assume contiguous [B,H,S,D] with S a multiple of 128 and keep their instruction
 // stream free of all that.  ALIBI (GENERAL only) subtracts slope[h] * |position - key| from the scaled score.
-// Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B
-// operands loaded once into registers, the walked tiles are A operands streamed through LDS by direct
-// global->LDS loads, and an accumulator tile is already laid out as the B operand of the next product.
+// DROPOUT (GENERAL only) replays the forward pass's keep decisions from (seed, head, query position, key).
+// Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the
+// lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B operands loaded once into
+// registers, the walked tiles are A operands streamed through LDS by direct global->LDS loads, and an
+// accumulator tile is already laid out as the B operand of the next product.
 // A walked tile that is needed both row-wise (ds_read_b128) and transposed (ds_read_b64_tr_b16) sits in LDS
 // once, under a swizzle that is bank-conflict-free for both.
 #ifndef FA_BWD_KERNEL_IMPL_H
