@@ -49,6 +49,7 @@ EXPORTED_SYMBOLS = (
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
     "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_algorithmic_flops",
+    "fa_bwd_sched_query_tile_range", "fa_bwd_sched_classify",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
     "fa_event_elapsed_ms", "fa_event_destroy",
@@ -149,6 +150,9 @@ def lib():
         L.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
         L.fa_bwd_algorithmic_flops.restype = ctypes.c_double
         L.fa_bwd_algorithmic_flops.argtypes = [ctypes.c_int] * 7
+        L.fa_bwd_sched_query_tile_range.restype = None
+        L.fa_bwd_sched_query_tile_range.argtypes = [ctypes.c_int] * 7 + [ctypes.POINTER(ctypes.c_int)] * 2
+        L.fa_bwd_sched_classify.argtypes = [ctypes.c_int] * 8
         L.fa_dropout_keep.argtypes = [ctypes.c_ulonglong, ctypes.c_longlong, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib

@@ -530,6 +530,24 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
 }
 
+void fa_bwd_sched_query_tile_range(int S, int S_kv, int is_causal, int window_left, int window_right,
+                                   int k_begin, int rows, int *tile_lo, int *tile_hi)
+{
+    const int Sk = S_kv > 0 ? S_kv : S, off = Sk - S;
+    int L, R;
+    fa_mask_bounds(S + Sk, is_causal, window_left, window_right, &L, &R);
+    fa_tile_range(S, 64, R + off, L - off, k_begin, rows, tile_lo, tile_hi);
+}
+
+int fa_bwd_sched_classify(int S, int S_kv, int is_causal, int window_left, int window_right,
+                          int k_begin, int rows, int tile)
+{
+    const int Sk = S_kv > 0 ? S_kv : S, off = Sk - S;
+    int L, R;
+    fa_mask_bounds(S + Sk, is_causal, window_left, window_right, &L, &R);
+    return fa_tile_class(64, R + off, L - off, k_begin, rows, tile);
+}
+
 // Five products over the unmasked pairs (the forward has two).  Square problems only, like fa_algorithmic_flops.
 double fa_bwd_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
 {

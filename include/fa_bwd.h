@@ -53,6 +53,14 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p);
 /* Enqueues two kernels on `stream` (dQ and the row sums of dO*O, then dK and dV) and returns without
  * synchronising.  No atomics: the same inputs give the same bits on every run. */
 int fa_bwd(const fa_bwd_params *p, void *stream);
+/* Host mirror of the arithmetic with which the key-owning kernel finds its work (csrc/fa_sched.h with the two
+ * sides of the mask exchanged and shifted by S_kv - S): the inclusive range of 64-query tiles that contain a
+ * query seeing at least one of the keys [k_begin, k_begin + rows), lo > hi when there is none; and the class of
+ * one such tile (0 = no pair visible, 2 = all visible, 1 = mixed).  S_kv = 0 means S. */
+void fa_bwd_sched_query_tile_range(int S, int S_kv, int is_causal, int window_left, int window_right,
+                                   int k_begin, int rows, int *tile_lo, int *tile_hi);
+int fa_bwd_sched_classify(int S, int S_kv, int is_causal, int window_left, int window_right,
+                          int k_begin, int rows, int tile);
 /* Algorithmic FLOPs of the backward pass: 10 * B * N * d * pairs (five products over the unmasked pairs). */
 double fa_bwd_algorithmic_flops(int B, int N, int S, int d, int is_causal, int window_left, int window_right);
 

@@ -205,3 +205,43 @@ def test_dropout_host_mirror(fa):
         want = numpy_keep_mask(seed, bh, 80, thr)
         got = np.array([[L.fa_dropout_keep(seed, bh, i, j, thr) for j in range(80)] for i in range(80)], dtype=bool)
         assert np.array_equal(got, want)
+
+
+def test_backward_key_block_schedule_against_brute_force(fa):
+    """The key-owning backward kernel walks the query tiles that see its keys; its range and tile classes come
+    from the forward's arithmetic with the mask's two sides exchanged and shifted by S_kv - S.  Checked here
+    against the mask predicate itself, pair by pair, for lengths that differ either way."""
+    L = fa.lib()
+    rng = np.random.default_rng(5)
+    cases = [(256, 0, 1, -1, -1), (300, 0, 1, 37, -1), (200, 456, 1, -1, -1), (320, 70, 1, 20, -1), (129, 513, 0, 10, 10),
+             (192, 64, 1, -1, -1), (257, 100, 0, -1, -1), (64, 640, 0, 100, 3), (500, 500, 0, -1, 33), (70, 300, 1, 0, -1)]
+    for S, S_kv, causal, wl, wr in cases:
+        Sk = S_kv or S
+        pos = np.arange(S)[:, None] + (Sk - S)
+        j = np.arange(Sk)[None, :]
+        vis = np.ones((S, Sk), dtype=bool)
+        if causal:
+            vis &= j <= pos
+        if wl >= 0:
+            vis &= pos - j <= wl
+        if wr >= 0 and not causal:
+            vis &= j - pos <= wr
+        n_tiles = (S + 63) // 64
+        for rows in (32, 256):
+            for k_begin in range(0, Sk, rows):
+                n = min(rows, Sk - k_begin)
+                block = vis[:, k_begin:k_begin + n]
+                lo, hi = ctypes.c_int(), ctypes.c_int()
+                L.fa_bwd_sched_query_tile_range(S, S_kv, causal, wl, wr, k_begin, n, ctypes.byref(lo), ctypes.byref(hi))
+                seen = [t for t in range(n_tiles) if block[64 * t:64 * t + 64].any()]
+                if not seen:
+                    assert lo.value > hi.value, (S, S_kv, causal, wl, wr, k_begin)
+                    continue
+                # the band is contiguous: the range is exactly the tiles with a visible pair
+                assert (lo.value, hi.value) == (seen[0], seen[-1]), (S, S_kv, causal, wl, wr, k_begin, rows)
+                for t in range(lo.value, hi.value + 1):
+                    if 64 * t + 64 > S:
+                        continue                      # the ragged last tile is always treated as mixed by the kernel
+                    sub = block[64 * t:64 * t + 64]
+                    cls = L.fa_bwd_sched_classify(S, S_kv, causal, wl, wr, k_begin, n, t)
+                    assert cls == (2 if sub.all() else 0 if not sub.any() else 1), (S, S_kv, causal, wl, wr, k_begin, rows, t)
