@@ -247,6 +247,8 @@ TINY = [
     (1, 2, 2, 257, 100, 128, 1, True, 40, -1),        # causal window, queries before the first key, bf16
     (1, 9, 3, 129, 513, 64, 0, False, 10, 10),        # nine heads: the last group of eight is a single head
     (3, 1, 1, 64, 64, 128, 0, True, 0, -1),           # window 0: every query sees only itself
+    (16, 24, 8, 128, 128, 64, 0, True, -1, -1),       # many small heads: 384 work items of one block each
+    (1, 2, 2, 2048, 2048, 128, 1, True, 256, -1),     # a sliding window much shorter than the sequence, bf16
 ]
 
 
