@@ -26,6 +26,7 @@
 #define FA_BWD_KERNEL_IMPL_H
 #include "fa_fwd_kernel_impl.h"
 #include "fa_bwd_args.h"
+#include "fa_bwd_layout.h"
 
 namespace {
 
@@ -37,16 +38,6 @@ constexpr float kLog2e = 1.44269504088896340736f;
 // (`__builtin_bit_cast(float, v[e])`) reads element 0 whatever e is with this compiler.
 __device__ __forceinline__ float as_f32(uint32_t w) { return __builtin_bit_cast(float, w); }
 
-// One 16-byte-chunk swizzle that serves both read patterns of a walked tile, so that the tile sits in LDS once:
-// ds_read_b128 by 16 lanes on 16 consecutive rows and one logical chunk needs 16 different chunk positions
-// (a bijection of the row's low bits), ds_read_b64_tr_b16 by 32 lanes on 4 consecutive rows x 4 consecutive
-// chunks needs the 4 rows in 4 different 64-byte groups (the two high bits follow the row's low bits).
-// Invariant under row += 16, not under row += 8.
-template <int CPR> __device__ __forceinline__ int u_swz(int row)
-{
-    return CPR == 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
-}
-
 // per-lane LDS addresses of the two read patterns in the stage being read; everything else about a fragment
 // (which of the stage's tiles, which 32-row block, which 16-row slice) is an immediate offset of the read
 template <int D> struct TileReader {
@@ -55,17 +46,12 @@ template <int D> struct TileReader {
     uint32_t tr_addr[DB][2];    // ds_read_b64_tr_b16: A operand rows = head dim (block db), k = 16 tile rows (two reads of 8)
     __device__ __forceinline__ void init(int lane, uint32_t stage_base)
     {
-        const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) row_addr[s] = stage_base + (uint32_t)(l32 * ROWB + (((2 * s + half) ^ u_swz<CPR>(l32)) << 4));
-        const int row0 = 4 * half + (l16 >> 2), dq = l32 >> 4, c4 = l16 & 3;
+        for (int s = 0; s < KS; ++s) row_addr[s] = stage_base + (uint32_t)fa_bwd_row_read(D, lane, s);
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int hi = 0; hi < 2; ++hi) {
-                const int c = 4 * db + 2 * dq + (c4 >> 1), row = row0 + 8 * hi;
-                tr_addr[db][hi] = stage_base + (uint32_t)(row * ROWB + ((c ^ u_swz<CPR>(row)) << 4) + ((c4 & 1) << 3));
-            }
+            for (int hi = 0; hi < 2; ++hi) tr_addr[db][hi] = stage_base + (uint32_t)fa_bwd_tr_read(D, lane, db, hi);
     }
     // move to another stage of the ring (delta in bytes, wave-uniform)
     __device__ __forceinline__ void advance(int delta)
@@ -97,8 +83,7 @@ template <int D> struct TileLoader {
         wave = wave_; lane = lane_;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
-            const int P = (i * kBwdWaves + wave) * 64 + lane, row = P / CPR, pos = P % CPR;
-            g[i] = (uint32_t)(row * row_bytes + ((pos ^ u_swz<CPR>(row)) << 4));
+            g[i] = (uint32_t)fa_bwd_load_source(D, (i * kBwdWaves + wave) * 64 + lane, row_bytes);
         }
     }
     __device__ __forceinline__ void load(const uint16_t *tile_src, uint32_t lds_tile) const
@@ -118,7 +103,7 @@ template <int D> struct TileLoader {
         for (int i = 0; i < IPW; ++i) {
             const int P = (i * kBwdWaves + wave) * 64 + ln, row = P / CPR, pos = P % CPR;
             const int src_row = row < valid ? row : valid - 1;
-            dma_16(reinterpret_cast<const char *>(tile_src), (uint32_t)(src_row * row_bytes + ((pos ^ u_swz<CPR>(row)) << 4)),
+            dma_16(reinterpret_cast<const char *>(tile_src), (uint32_t)(src_row * row_bytes + ((pos ^ fa_u_swz(CPR, row)) << 4)),
                    lds_tile + (i * kBwdWaves + wave) * 1024);
         }
     }

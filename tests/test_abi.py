@@ -245,3 +245,17 @@ def test_backward_key_block_schedule_against_brute_force(fa):
                     sub = block[64 * t:64 * t + 64]
                     cls = L.fa_bwd_sched_classify(S, S_kv, causal, wl, wr, k_begin, n, t)
                     assert cls == (2 if sub.all() else 0 if not sub.any() else 1), (S, S_kv, causal, wl, wr, k_begin, rows, t)
+
+
+def test_backward_lds_layout_arithmetic_on_the_host():
+    """The header the backward kernels take their LDS addresses from compiles as C: what the direct loads write
+    is what both read patterns find, every address stays inside the tile, and neither pattern has a bank
+    conflict (tests/c/check_bwd_layout.c)."""
+    import subprocess
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        exe = os.path.join(tmp, "check_bwd_layout")
+        subprocess.run(["gcc", "-O1", "-Wall", "-Wextra", "-I", os.path.join(REPO, "flash-attn-rtx5060_amd", "csrc"),
+                        os.path.join(REPO, "tests", "c", "check_bwd_layout.c"), "-o", exe], check=True)
+        out = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
+    assert out.returncode == 0, out.stdout
