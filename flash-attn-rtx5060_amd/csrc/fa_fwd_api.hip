@@ -309,10 +309,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         a.v_bs = eff[2][0]; a.v_hs = eff[2][1]; a.v_rs = (int)eff[2][2];
         a.o_bs = eff[3][0]; a.o_hs = eff[3][1]; a.o_rs = (int)eff[3][2];
     }
-    // The 8-wave instantiations for general layouts come back from the compiler with 270-350 bytes of spills whose
-    // reloads wait on the tile loads in flight; the 4-wave ones have none (c3's shape stored [B,S,H,D]: 615 against
-    // 904 TFLOP/s).  With dropout both shapes spill and the 8-wave one is the faster (473 against 375).
-    const int waves = (general && !(p->dropout_prob > 0.0f)) ? 4 : waves_for(p->B, p->N, p->S);
+    const int waves = waves_for(p->B, p->N, p->S);
     const int block_rows = 32 * waves;
     a.n_qblocks = a.pack > 1 ? 1 : (p->S + block_rows - 1) / block_rows;
     const int s_max = a.Sk > p->S ? a.Sk : p->S;        // stands in for "unbounded"

@@ -910,13 +910,16 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 // shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
 // (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
 // answers it with about 500 AGPR<->VGPR moves per tile.)
+// (The 8-wave general instantiations get two LDS stages instead of three: with three they come back from the
+// compiler with 270-350 bytes of spills whose reloads wait on the tile loads in flight -- c3's shape stored
+// [B,S,H,D] ran at 615 TFLOP/s, with two stages nothing spills and it runs at 940.)
 template <bool GENERAL, bool DROPOUT>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, 3>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : 3)>(a, grid, stream); \
         return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)

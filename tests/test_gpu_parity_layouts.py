@@ -117,9 +117,9 @@ def test_headline_shape_in_bshd_layout(fa, oracle):
                  lse.cpu().numpy().reshape(-1)[rows], lse_ref)
     print("c3 BSHD", err)
     assert_within(err, 0, "c3 in BSHD layout")
-    # The contiguous layout runs the 256-row workgroup, this one the 128-row one: the same products and
-    # exponentials, but the row sums are added up in another order in the iterations that fill and drain the
-    # pipeline, so the results agree to the last bits rather than bit for bit.
+    # The contiguous layout runs with three LDS stages, this one with two: the same products and exponentials,
+    # but the row sums are added up in another order in the iterations that fill and drain the pipeline, so the
+    # results agree to the last bits rather than bit for bit.
     o2, lse2 = fa.flash_attention_forward(to_torch(q, 0), to_torch(k, 0), to_torch(v, 0), causal=True)
     torch.cuda.synchronize()
     assert float((o.contiguous().float() - o2.float()).abs().max()) <= 2.0 ** -9          # one fp16 ulp at |O| < 4
