@@ -188,6 +188,10 @@ def main():
                     help="override the standard deviation of the inputs (0 = all-zero tensors: the same instruction "
                          "stream without data-dependent switching power; not the headline metric)")
     ap.add_argument("--dropout", type=float, default=0.0, help="dropout probability (not the headline metric), seed 48")
+    ap.add_argument("--layout", default="bhsd", choices=("bhsd", "bshd"),
+                    help="bshd: the same values stored [B,S,H,D] and passed as strided views (not the headline metric)")
+    ap.add_argument("--kv-heads", type=int, default=0, metavar="N",
+                    help="K and V with N heads, shared by groups of query heads (not the headline metric)")
     ap.add_argument("--backward", action="store_true", help="time the backward pass on the workload's shape (not the headline metric)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
@@ -214,7 +218,13 @@ def main():
         sigma = args.sigma
     shape = (B, H, S, D)
     q, k, v = make_inputs(fa, shape, dtype, seed, sigma, frac, mult)
+    if args.kv_heads:
+        if H % args.kv_heads:
+            sys.exit("bench.py: --kv-heads must divide the number of heads")
+        k, v = (np.ascontiguousarray(x[:, :args.kv_heads]) for x in (k, v))
     tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    if args.layout == "bshd":
+        tq, tk, tv = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv))
     out = torch.empty_like(tq)
     lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
 
@@ -251,7 +261,8 @@ def main():
     kernel_tflops = flops / (avg_kernel_ms * 1e-3) / 1e12
     algo_bytes = 4 * B * H * S * D * 2 + B * H * S * 4
 
-    variant = args.alibi or args.dropout > 0 or args.sigma is not None       # not the headline problem
+    variant = (args.alibi or args.dropout > 0 or args.sigma is not None or args.layout != "bhsd"
+               or args.kv_heads)                                                  # not the headline problem
     result = {
         "metric": ("attn fwd TFLOPS + % of fp16 MFMA peak, hd128 causal seq 8192, 1 GPU" if args.workload == "c3" and not variant
                    else f"attn fwd TFLOPS + % of MFMA peak, workload {args.workload}, 1 GPU"),
@@ -261,11 +272,13 @@ def main():
         "config": {"workload": f"{args.workload}: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D} "
                                f"{'causal' if causal else 'non-causal'}{f' window_left {wl}' if wl >= 0 else ''}, "
                                f"scale 1/sqrt({D}), fp32 accumulate, O + logsumexp{', ALiBi' if args.alibi else ''}"
-                               f"{f', dropout {args.dropout}' if args.dropout else ''}",
+                               f"{f', dropout {args.dropout}' if args.dropout else ''}"
+                               f"{', stored [B,S,H,D]' if args.layout == 'bshd' else ''}"
+                               f"{f', {args.kv_heads} K/V heads' if args.kv_heads else ''}",
                    "seed": seed, "sigma": sigma, "algorithmic_flops": flops, "algorithmic_bytes": algo_bytes},
         "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None if (args.alibi or args.dropout) else MEASURED_HBM_BYTES.get(args.workload),
+                     "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None if variant else MEASURED_HBM_BYTES.get(args.workload),
                      "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_median": round(float(np.median(kernel_ms)), 5),
                      "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
     }
@@ -274,8 +287,10 @@ def main():
     if args.check_rows > 0:
         import oracle_binding as ob
         rows = sample_rows(shape, args.check_rows, seed)
-        o_ref, lse_ref = ob.rows(q, k, v, rows, dtype, None, causal, wl, -1, slopes, dropout=drop)
-        err = errors(ob.to_f32(from_torch(out), dtype).reshape(-1, D)[rows], ob.to_f32(o_ref, dtype),
+        rep = H // k.shape[1]
+        kf, vf = (np.repeat(x, rep, axis=1) if rep > 1 else x for x in (k, v))
+        o_ref, lse_ref = ob.rows(q, kf, vf, rows, dtype, None, causal, wl, -1, slopes, dropout=drop)
+        err = errors(ob.to_f32(from_torch(out.contiguous()), dtype).reshape(-1, D)[rows], ob.to_f32(o_ref, dtype),
                      lse.cpu().numpy().reshape(-1)[rows], lse_ref)
         err["rows_checked"] = int(len(rows))
         grow = 256.0 / (256 - drop[0])      # kept probabilities, and their rounding differences, are scaled by this
