@@ -117,7 +117,13 @@ def backward_bench(args):
     B, H, S, D, dtype, causal, wl, sigma, frac, mult, seed = WORKLOADS[args.workload]
     q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed, sigma, frac, mult)
     do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed + 1000)
+    if args.kv_heads:
+        if H % args.kv_heads:
+            sys.exit("bench.py: --kv-heads must divide the number of heads")
+        k, v = (np.ascontiguousarray(x[:, :args.kv_heads]) for x in (k, v))
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    if args.layout == "bshd":
+        tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
     kw = dict(causal=causal, window_left=wl, dropout_prob=args.dropout, seed=48)
     o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
     grads = [None]
@@ -137,7 +143,7 @@ def backward_bench(args):
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     gpu_ms = e0.elapsed_time(e1) / args.steps
     flops = fa.lib().fa_bwd_algorithmic_flops(B, H, S, D, int(causal), wl, -1)
-    # parity on the last head
+    # parity on the last head (with grouped K/V heads: the last query head alone, so only dQ is comparable)
     qf, kf, vf = (t[-1, -1].float().requires_grad_(True) for t in (tq, tk, tv))
     i = torch.arange(S, device="cuda")
     vis = torch.ones((S, S), dtype=torch.bool, device="cuda")
@@ -153,7 +159,7 @@ def backward_bench(args):
         pm = pm * torch.from_numpy(numpy_keep_mask(48, B * H - 1, S, thr).astype(np.float32) * (256.0 / (256 - thr))).cuda()
     (pm @ vf).backward(tdo[-1, -1].float())
     err = {}
-    for name, got, want in zip(("dQ", "dK", "dV"), grads[0], (qf.grad, kf.grad, vf.grad)):
+    for name, got, want in list(zip(("dQ", "dK", "dV"), grads[0], (qf.grad, kf.grad, vf.grad)))[:1 if args.kv_heads else 3]:
         d = got[-1, -1].float() - want
         err[name] = {"rel_l2": float(d.norm() / want.norm()), "max_abs": float(d.abs().max()), "max_ref": float(want.abs().max())}
     tf = flops / (wall_ms * 1e-3) / 1e12
@@ -163,11 +169,13 @@ def backward_bench(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
         "config": {"workload": f"{args.workload} backward: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D}"
                                f"{' causal' if causal else ''}{f' window_left {wl}' if wl >= 0 else ''}"
-                               f"{f' dropout {args.dropout}' if args.dropout > 0 else ''}",
+                               f"{f' dropout {args.dropout}' if args.dropout > 0 else ''}"
+                               f"{', stored [B,S,H,D]' if args.layout == 'bshd' else ''}"
+                               f"{f', {args.kv_heads} K/V heads' if args.kv_heads else ''}",
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 else None,
+                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads else None,
                      "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_dq + fa_bwd_dkdv"},
         "parity_vs_torch_fp32_one_head": err}))
 
