@@ -124,3 +124,30 @@ def test_headline_shape_in_bshd_layout(fa, oracle):
     torch.cuda.synchronize()
     assert float((o.contiguous().float() - o2.float()).abs().max()) <= 2.0 ** -9          # one fp16 ulp at |O| < 4
     assert float((lse - lse2).abs().max()) <= 1e-5
+
+
+@pytest.mark.parametrize("shape,Hk,S_real", [((2, 16, 1024, 128), 4, 1024), ((4, 32, 512, 64), 32, 500), ((1, 64, 2048, 128), 8, 2048)])
+def test_general_layouts_under_every_schedule(fa, oracle, shape, Hk, S_real):
+    """[B,S,H,D] storage with grouped K/V heads (and a ragged length) through the three ways of walking the work
+    list, with both workgroup shapes occurring among the cases: sampled rows against the oracle, and the same
+    bits from every schedule."""
+    import torch
+    B, H, _, D = shape
+    S = S_real
+    q, _, _ = make_inputs(fa, (B, H, S, D), 0, seed=61)
+    _, k, v = make_inputs(fa, (B, Hk, S, D), 0, seed=62)
+    tq, tk, tv = (to_torch(x, 0).transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v))
+    rows = sample_rows((B, H, S, D), 512, 61)
+    rep = H // Hk
+    o_ref, lse_ref = oracle.rows(q, np.repeat(k, rep, axis=1), np.repeat(v, rep, axis=1), rows, 0, None, True, -1, -1)
+    outs = []
+    for sched in (fa.FA_SCHED_DISPATCH, fa.FA_SCHED_PERSISTENT, fa.FA_SCHED_QUEUE):
+        o, lse = fa.flash_attention_forward(tq, tk, tv, causal=True, sched=sched)
+        torch.cuda.synchronize()
+        err = errors(oracle.to_f32(from_torch(o.contiguous()), 0).reshape(-1, D)[rows], oracle.to_f32(o_ref, 0),
+                     lse.cpu().numpy().reshape(-1)[rows], lse_ref)
+        print(shape, Hk, S, "sched", sched, err)
+        assert_within(err, 0, f"general layout, schedule {sched}")
+        outs.append((o, lse))
+    for o, lse in outs[1:]:
+        assert torch.equal(o.view(torch.int16), outs[0][0].view(torch.int16)) and torch.equal(lse, outs[0][1])
