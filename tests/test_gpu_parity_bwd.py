@@ -289,3 +289,22 @@ def test_autograd_wrapper_trains_like_torch_attention(fa):
         print("autograd wrapper", name, err, flush=True)
         # the loss gradient dO = w + out is itself rounded to fp16 on the way into fa_bwd
         assert err["nonfinite"] == 0 and err["rel_l2"] <= 2e-3 and err["max_abs"] <= 4e-3 * max(1.0, err["max_ref"]), (name, err)
+
+
+def test_gradients_with_outlier_query_rows(fa, oracle):
+    """c5's input recipe on a small shape: sigma 0.5 and a seeded 5 % of the query rows multiplied by 8, so that
+    some rows have one dominant key (P close to one-hot, large logsumexp) next to ordinary ones."""
+    import torch
+    shape, dtype = (1, 4, 512, 128), 0
+    q, k, v = make_inputs(fa, shape, dtype, 31, 0.5, 0.05, 8.0)
+    do, _, _ = make_inputs(fa, shape, dtype, seed=32)
+    dq_ref, dk_ref, dv_ref = oracle.bwd_f64(q, k, v, do, dtype, None, True, -1, -1)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=True)
+    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=True)
+    torch.cuda.synchronize()
+    assert float(lse.max()) > 8.0          # the outlier rows are there
+    for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
+        err = grad_errors(oracle.to_f32(from_torch(got), dtype), want)
+        print("outlier rows", name, err, flush=True)
+        check(err, dtype, name)
