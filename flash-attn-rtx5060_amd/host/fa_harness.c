@@ -17,7 +17,7 @@
  * usage: fa_harness [--config c1..c5] [--B n --N n --S n --d n] [--bf16]
  *                   [--causal] [--window-left n] [--window-right n]
  *                   [--scale x] [--seed n] [--sigma x] [--iters n] [--warmup n]
- *                   [--threads n] [--dump prefix] [--no-lse]
+ *                   [--threads n] [--dump prefix] [--no-lse] [--backward]
  */
 #include <math.h>
 #include <stdio.h>
@@ -25,6 +25,7 @@
 #include <string.h>
 
 #include "fa_fwd.h"
+#include "fa_bwd.h"
 #include "fa_inputs.h"
 
 #define PEAK_TFLOPS 2516.6 /* 256 CU x 4096 FLOP/clk x 2.4 GHz, dense fp16 = bf16 */
@@ -36,6 +37,7 @@ typedef struct {
     double row_fraction;
     float row_mult;
     const char *dump;
+    int backward;       /* also run fa_bwd on a seeded dO (the reference has no backward pass) */
     const char *name;
 } cfg_t;
 
@@ -107,6 +109,7 @@ int main(int argc, char **argv)
         else if (!strcmp(a, "--threads")) { NEED_VALUE(); c.threads = atoi(v); }
         else if (!strcmp(a, "--dump")) { NEED_VALUE(); c.dump = v; }
         else if (!strcmp(a, "--no-lse")) c.lse = 0;
+        else if (!strcmp(a, "--backward")) c.backward = 1;
         else if (!strcmp(a, "--alibi")) c.alibi = 1;
         else if (!strcmp(a, "--dropout")) { NEED_VALUE(); c.dropout = (float)atof(v); }
         else { fprintf(stderr, "unknown argument %s\n", a); return 2; }
@@ -193,12 +196,67 @@ int main(int argc, char **argv)
            flops / med / 1e9 / PEAK_TFLOPS, bad);
 
     int rc = bad ? 4 : 0;
+    uint16_t *hg[4] = {NULL, NULL, NULL, NULL};      /* dO, dQ, dK, dV on the host */
+    if (c.backward) {
+        /* gradients of sum(dO * O) through fa_bwd, with dO from the same generator (tensor slot of Q, seed + 1000):
+           a second JSON line; the forward pass above has left O and the logsumexp on the device */
+        if (!c.lse) { fprintf(stderr, "--backward needs the logsumexp (drop --no-lse)\n"); return 2; }
+        void *dg[4] = {NULL, NULL, NULL, NULL}, *ws = NULL;
+        for (int t = 0; t < 4; ++t) {
+            hg[t] = malloc(bytes);
+            if (!hg[t] || check(fa_dev_malloc(&dg[t], bytes), "alloc gradient")) return 1;
+        }
+        if (fa_fill_normal(hg[0], rows, c.d, c.bf16, c.seed + 1000, FA_TENSOR_Q, 1.0f, 0.0, 1.0f, c.threads) ||
+            check(fa_dev_h2d(dg[0], hg[0], bytes), "H2D dO")) return 1;
+        fa_bwd_params b;
+        memset(&b, 0, sizeof(b));
+        b.Q = dq; b.K = dk; b.V = dv; b.O = dO; b.dO = dg[0]; b.L = (const float *)dl;
+        b.dQ = dg[1]; b.dK = dg[2]; b.dV = dg[3];
+        b.B = c.B; b.N = c.N; b.S = c.S; b.d = c.d;
+        b.softmax_scale = c.scale;
+        b.window_size_left = c.wl; b.window_size_right = c.wr;
+        b.dtype = p.dtype; b.is_causal = c.causal;
+        b.alibi_slopes_ptr = p.alibi_slopes_ptr;
+        b.dropout_prob = p.dropout_prob; b.seed = p.seed;
+        b.workspace_bytes = fa_bwd_workspace_bytes(&b);
+        if (check(fa_dev_malloc(&ws, (size_t)b.workspace_bytes), "alloc workspace")) return 1;
+        b.workspace = ws;
+        for (int i = 0; i < c.warmup; ++i)
+            if (check(fa_bwd(&b, NULL), "backward warm-up launch")) return 1;
+        if (check(fa_dev_sync(), "sync")) return 1;
+        for (int i = 0; i < c.iters; ++i) {
+            if (check(fa_event_record(e0, NULL), "record") || check(fa_bwd(&b, NULL), "backward launch") ||
+                check(fa_event_record(e1, NULL), "record") || check(fa_event_sync(e1), "event sync") ||
+                check(fa_event_elapsed_ms(e0, e1, &ms[i]), "elapsed")) return 1;
+        }
+        size_t bad_g = 0;
+        for (int t = 1; t < 4; ++t) {
+            if (check(fa_dev_d2h(hg[t], dg[t], bytes), "D2H gradient")) return 1;
+            for (size_t i = 0; i < elems; ++i) {
+                const float x = c.bf16 ? fa_bf16_bits_to_f32(hg[t][i]) : fa_f16_bits_to_f32(hg[t][i]);
+                if (!isfinite(x)) ++bad_g;
+            }
+        }
+        qsort(ms, (size_t)c.iters, sizeof(float), cmp_float);
+        const double bmed = ms[c.iters / 2], bbest = ms[0];
+        const double bflops = fa_bwd_algorithmic_flops(c.B, c.N, c.S, c.d, c.causal, c.wl, c.wr);
+        printf("{\"config\": \"%s backward\", \"iters\": %d, \"ms_median\": %.6f, \"ms_min\": %.6f, \"algorithmic_flops\": %.6e, "
+               "\"tflops_median\": %.3f, \"tflops_best\": %.3f, \"frac_of_peak_median\": %.4f, \"nonfinite_gradients\": %zu}\n",
+               c.name, c.iters, bmed, bbest, bflops, bflops / bmed / 1e9, bflops / bbest / 1e9, bflops / bmed / 1e9 / PEAK_TFLOPS, bad_g);
+        if (bad_g) rc |= 4;
+        for (int t = 0; t < 4; ++t) fa_dev_free(dg[t]);
+        fa_dev_free(ws);
+    }
     if (c.dump) {
         rc |= dump_file(c.dump, "q.bin", hq, bytes) | dump_file(c.dump, "k.bin", hk, bytes) |
               dump_file(c.dump, "v.bin", hv, bytes) | dump_file(c.dump, "o.bin", ho, bytes);
         if (c.lse) rc |= dump_file(c.dump, "lse.bin", hl, rows * sizeof(float));
         if (c.alibi) rc |= dump_file(c.dump, "slopes.bin", hs, (size_t)c.N * sizeof(float));
+        if (c.backward)
+            rc |= dump_file(c.dump, "do.bin", hg[0], bytes) | dump_file(c.dump, "dq.bin", hg[1], bytes) |
+                  dump_file(c.dump, "dk.bin", hg[2], bytes) | dump_file(c.dump, "dv.bin", hg[3], bytes);
     }
+    for (int t = 0; t < 4; ++t) free(hg[t]);
     fa_event_destroy(e0); fa_event_destroy(e1);
     fa_dev_free(dq); fa_dev_free(dk); fa_dev_free(dv); fa_dev_free(dO); fa_dev_free(dl);
     if (ds) fa_dev_free(ds);

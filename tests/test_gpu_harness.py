@@ -46,3 +46,34 @@ def test_harness_output_matches_oracle(fa, oracle, tmp_path, args, shape, dtype,
     o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, causal, wl, -1, slopes, dropout=drop)
     err = errors(oracle.to_f32(o[rows], dtype), oracle.to_f32(o_ref, dtype), lse[rows], lse_ref)
     assert_within(err, dtype, f"harness {args}")
+
+
+@pytest.mark.parametrize("args,shape,dtype,causal,wl,seed", [
+    (["--config", "c1"], (1, 4, 256, 64), 0, False, -1, 27),
+    (["--B", "1", "--N", "3", "--S", "500", "--d", "128", "--causal", "--alibi", "--dropout", "0.1", "--seed", "9"],
+     (1, 3, 500, 128), 0, True, -1, 9),
+])
+def test_harness_backward_matches_gradient_oracle(fa, oracle, tmp_path, args, shape, dtype, causal, wl, seed):
+    """--backward: fa_bwd called from plain C on the forward pass's O and logsumexp; the dumped gradients against
+    the fp64 gradient oracle (dO comes from the same seeded generator, seed + 1000)."""
+    prefix = str(tmp_path / "run")
+    proc = subprocess.run([fa.HARNESS_PATH, *args, "--backward", "--iters", "2", "--warmup", "1", "--dump", prefix],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    lines = proc.stdout.strip().splitlines()
+    report = json.loads(lines[-1])
+    B, H, S, D = shape
+    assert report["config"].endswith("backward") and report["nonfinite_gradients"] == 0
+    assert report["algorithmic_flops"] == pytest.approx(2.5 * json.loads(lines[-2])["algorithmic_flops"])
+    q, k, v, do = (np.fromfile(f"{prefix}.{t}.bin", dtype=np.uint16).reshape(shape) for t in ("q", "k", "v", "do"))
+    do2, _, _ = make_inputs(fa, shape, dtype, seed + 1000)
+    assert np.array_equal(do, do2)
+    slopes = np.fromfile(f"{prefix}.slopes.bin", dtype=np.float32) if "--alibi" in args else None
+    drop = (fa.lib().fa_dropout_threshold(0.1), 48) if "--dropout" in args else (0, 0)
+    want = oracle.bwd_f64(q, k, v, do, dtype, None, causal, wl, -1, slopes, dropout=drop)
+    grow = 256.0 / (256 - drop[0])
+    for name, ref in zip(("dq", "dk", "dv"), want):
+        got = oracle.to_f32(np.fromfile(f"{prefix}.{name}.bin", dtype=np.uint16).reshape(shape), dtype).astype(np.float64)
+        rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+        print("harness backward", args[:2], name, rel)
+        assert np.isfinite(got).all() and rel <= 1e-3 * grow, (name, rel)
