@@ -1,0 +1,96 @@
+"""Forty seeded random configurations (lengths, heads, head groups, head dim, dtype, masks, ALiBi, dropout, storage order)
+through fa_fwd and fa_bwd, compared with an explicit fp32 attention and its autograd gradients in torch on the
+GPU.  The oracle-based tests pin the arithmetic on chosen cases; this sweep is there for the index arithmetic of
+combinations nobody chose."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def reference(q, k, v, do, causal, wl, wr, slopes, keep=None):
+    import torch
+    B, H, S, D = q.shape
+    Hk, Sk = k.shape[1], k.shape[2]
+    qf, kf, vf = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    kr, vr = (t.repeat_interleave(H // Hk, dim=1) for t in (kf, vf))
+    pos = torch.arange(S, device=q.device)[:, None] + (Sk - S)
+    j = torch.arange(Sk, device=q.device)[None, :]
+    vis = torch.ones((S, Sk), dtype=torch.bool, device=q.device)
+    if causal:
+        vis &= j <= pos
+    if wl >= 0:
+        vis &= pos - j <= wl
+    if wr >= 0 and not causal:
+        vis &= j - pos <= wr
+    s = torch.einsum("bhid,bhjd->bhij", qf, kr) * float(np.float32(1.0 / np.sqrt(D)))
+    if slopes is not None:
+        s = s - slopes[None, :, None, None] * (pos - j).abs()[None, None].float()
+    s = s.masked_fill(~vis, float("-inf"))
+    p = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
+    if keep is not None:            # [B,H,S,Sk] factors: 0 or 1/(1-p)
+        p = p * keep
+    o = torch.einsum("bhij,bhjd->bhid", p, vr)
+    (o * do.float()).sum().backward()
+    lse = torch.logsumexp(s, dim=-1)
+    return o.detach(), lse.detach(), qf.grad, kf.grad, vf.grad
+
+
+def test_random_configurations(fa):
+    import torch
+    rng = np.random.default_rng(20240607)
+    for case in range(40):
+        D = int(rng.choice([64, 128]))
+        dtype = torch.bfloat16 if rng.random() < 0.3 else torch.float16
+        Hk = int(rng.choice([1, 2, 3]))
+        H = Hk * int(rng.choice([1, 1, 2, 4]))
+        B = int(rng.integers(1, 3))
+        S = int(rng.integers(1, 700))
+        Sk = S if rng.random() < 0.5 else int(rng.integers(max(1, S - 100), S + 400))
+        causal = bool(rng.random() < 0.6)
+        wl = int(rng.integers(0, 300)) if rng.random() < 0.4 else -1
+        wr = int(rng.integers(0, 300)) if (not causal and rng.random() < 0.4) else -1
+        alibi = bool(rng.random() < 0.3)
+        bshd = bool(rng.random() < 0.5)
+        # dropout where the published decision function can be replayed by the numpy implementation as it stands
+        # (query positions from 0 up: not more queries than keys)
+        drop_p = float(rng.choice([0.1, 0.3, 0.5])) if (Sk >= S and rng.random() < 0.3) else 0.0
+        seed = int(rng.integers(1, 2 ** 40))
+        g = torch.Generator(device="cuda").manual_seed(1000 + case)
+
+        def make(h, s):
+            t = torch.randn((B, s, h, D) if bshd else (B, h, s, D), device="cuda", generator=g).to(dtype)
+            return t.transpose(1, 2) if bshd else t
+        q, do, k, v = make(H, S), make(H, S), make(Hk, Sk), make(Hk, Sk)
+        slopes = (torch.rand(H, device="cuda", generator=g) * 0.2 - 0.05).float().contiguous() if alibi else None
+        what = dict(case=case, B=B, H=H, Hk=Hk, S=S, Sk=Sk, D=D, dtype=str(dtype), causal=causal, wl=wl, wr=wr, alibi=alibi, bshd=bshd,
+                    dropout=drop_p)
+        print(what, flush=True)
+        kw = dict(causal=causal, window_left=wl, window_right=wr, alibi_slopes=slopes, dropout_prob=drop_p, seed=seed)
+        keep, grow = None, 1.0
+        if drop_p > 0:
+            from parity_util import numpy_keep_mask
+            thr = fa.lib().fa_dropout_threshold(drop_p)
+            grow = 256.0 / (256 - thr)
+            m = np.stack([numpy_keep_mask(seed, bh, Sk, thr)[Sk - S:] for bh in range(B * H)]).reshape(B, H, S, Sk)
+            keep = torch.from_numpy(m.astype(np.float32) * grow).cuda()
+        o, lse = fa.flash_attention_forward(q, k, v, **kw)
+        dq, dk, dv = fa.flash_attention_backward(q, k, v, o, lse, do, **kw)
+        torch.cuda.synchronize()
+        o_ref, lse_ref, dq_ref, dk_ref, dv_ref = reference(q, k, v, do, causal, wl, wr, slopes, keep)
+        half = dtype == torch.float16
+        assert bool(torch.isfinite(o.float()).all()), what
+        # (two ulps at |O| in [2, 4): the first rows of a causal head are computed in the reference verifier's
+        # arithmetic, which rounds every product to the storage type and sits up to an ulp away from exact fp32;
+        # an indexing mistake shows up as an error of order one)
+        assert float((o.float() - o_ref).abs().max()) <= (4e-3 if half else 3.2e-2) * grow, what
+        seen = torch.isfinite(lse_ref)
+        assert bool((lse[~seen] == float("-inf")).all()), what
+        if bool(seen.any()):
+            assert float((lse[seen] - lse_ref[seen]).abs().max()) <= (2e-3 if half else 8e-3), what
+        for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
+            d = got.float() - want
+            scale = max(1.0, float(want.abs().max()))
+            assert bool(torch.isfinite(got.float()).all()), (name, what)
+            assert float(d.abs().max()) <= (2e-3 if half else 1.6e-2) * scale * grow, (name, float(d.abs().max()), what)
+            assert float(d.norm()) <= (1e-3 if half else 8e-3) * grow * float(want.norm()) + 1e-5, (name, what)
