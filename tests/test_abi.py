@@ -259,3 +259,21 @@ def test_backward_lds_layout_arithmetic_on_the_host():
                         os.path.join(REPO, "tests", "c", "check_bwd_layout.c"), "-o", exe], check=True)
         out = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
     assert out.returncode == 0, out.stdout
+
+
+def test_key_split_suggestion_fills_the_device_once(fa):
+    """fa_fwd_suggest_splits: work items (K/V-head groups packed into one item when few queries sit behind long
+    keys) times splits should cover the 512 resident 4-wave workgroups of a 256-CU device once, with at least
+    four 64-key tiles per split; problems that fill the device by themselves are not split."""
+    L = fa.lib()
+
+    def suggest(B, N, Nk, S, S_kv):
+        p = fa.make_params(B, N, S, 128, 0x1000, 0x2000, 0x3000, 0x4000, causal=True, n_kv_heads=0 if Nk == N else Nk, S_kv=S_kv)
+        return L.fa_fwd_suggest_splits(ctypes.byref(p))
+    assert suggest(16, 32, 8, 1, 8192) == 4          # 128 packed items
+    assert suggest(4, 32, 32, 1, 32768) == 4         # 128 items
+    assert suggest(8, 32, 8, 4, 8192) == 8           # 64 packed items
+    assert suggest(1, 32, 8, 1, 65536) == 64         # 8 packed items
+    assert suggest(1, 8, 8, 1, 1024) == 4            # 8 items, capped by four tiles per split (16 tiles)
+    assert suggest(64, 32, 8, 1, 2048) == 1          # 512 packed items fill the device
+    assert suggest(2, 32, 32, 8192, 0) == 1          # a prefill-sized problem
