@@ -11,7 +11,10 @@
  * Pinning status (what checks this restatement against something other than
  * itself): the reference holds no golden vectors for this path, so the
  * oracle is pinned by closed forms, invariants, brute-force fp64 fixtures and
- * torch's scaled_dot_product_attention in tests/test_oracle.py.  Bit-exact
+ * torch's scaled_dot_product_attention in tests/test_oracle.py, and every
+ * rounding point of main.cu:193,259,261 (half product, p rounded to half,
+ * half product with v) by bit equality with an independent literal written in
+ * numpy float16 / torch bfloat16 arithmetic in the same file.  Bit-exact
  * agreement with the CUDA host `__half` operators of the reference build is
  * "parity unpinned": it follows from source semantics (float multiply of two
  * halves is exact, then one round-to-nearest-even) but no reference binary

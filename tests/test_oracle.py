@@ -94,6 +94,113 @@ def test_row_subset_equals_full():
     assert np.array_equal(lse_s, lse.reshape(-1)[idx])
 
 
+# ---------------------------------------------------------------- the verifier's roundings, by an independent literal
+# reference src/main.cu:189-263 restated with library half arithmetic only: numpy's float16 multiply IS the
+# half x half -> half product of main.cu:193 and :259 (numpy computes it in fp32 and rounds once), torch's CPU
+# bfloat16 multiply is the same for bf16; the sums are sequential fp32 adds in index order; expf is libm's.
+# Nothing here calls into oracle/; a rounding dropped on either side of the softmax changes output bits.
+def _libm_expf():
+    import ctypes.util
+    m = ctypes.CDLL(ctypes.util.find_library("m") or "libm.so.6")
+    m.expf.restype = ctypes.c_float
+    m.expf.argtypes = [ctypes.c_float]
+    return m.expf
+
+
+def _storage_mul(a32, b32, dtype):
+    """Elementwise product of storage-type values (given as float32), rounded to the storage type, widened."""
+    if dtype == F16:
+        return (a32.astype(np.float16) * b32.astype(np.float16)).astype(np.float32)
+    import torch
+    ta, tb = torch.from_numpy(np.ascontiguousarray(a32)).to(torch.bfloat16), torch.from_numpy(np.ascontiguousarray(b32)).to(torch.bfloat16)
+    return (ta * tb).to(torch.float32).numpy()
+
+
+def _storage_round(x32, dtype):
+    if dtype == F16:
+        return x32.astype(np.float16).astype(np.float32)
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x32)).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+def independent_verifier(qb, kb, vb, dtype, scale, causal, window):
+    """O bits [B,H,S,D] by the sequence of main.cu:176-266 (window < 0: none; symmetric, main.cu:220-229)."""
+    expf = _libm_expf()
+    B, H, S, D = qb.shape
+    q, k, v = (ob.to_f32(x, dtype) for x in (qb, kb, vb))
+    out = np.empty((B, H, S, D), dtype=np.uint16)
+    scale = np.float32(scale)
+    for b in range(B):
+        for h in range(H):
+            sc = np.zeros((S, S), dtype=np.float32)
+            for t in range(D):                                      # main.cu:192-194, fp32 sum in index order
+                sc = sc + _storage_mul(np.broadcast_to(q[b, h, :, t, None], (S, S)), np.broadcast_to(k[b, h, None, :, t], (S, S)), dtype)
+            sc = sc * scale                                          # main.cu:195
+            i, j = np.arange(S)[:, None], np.arange(S)[None, :]
+            if causal:
+                sc = np.where(j > i, np.float32(-np.inf), sc)        # main.cu:210-218
+            if window >= 0:
+                sc = np.where(np.abs(i - j) > window, np.float32(-np.inf), sc)   # main.cu:220-229
+            p = np.zeros((S, S), dtype=np.float32)
+            for r in range(S):                                      # main.cu:232-252
+                mx = np.float32(-np.inf)
+                for c in range(S):
+                    mx = max(mx, sc[r, c])
+                tot = np.float32(0.0)
+                e = np.zeros(S, dtype=np.float32)
+                for c in range(S):
+                    e[c] = np.float32(expf(float(np.float32(sc[r, c] - mx))))
+                    tot = np.float32(tot + e[c])
+                p[r] = e / tot
+            o = np.zeros((S, D), dtype=np.float32)
+            for c in range(S):                                      # main.cu:255-263: half(p) * v as a half product
+                o = o + _storage_mul(np.broadcast_to(p[:, c, None], (S, D)), np.broadcast_to(v[b, h, None, c, :], (S, D)), dtype)
+            out[b, h] = ob.from_f32(o, dtype)                        # main.cu:261
+    return out
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("causal,window", [(False, -1), (True, -1), (False, 3), (True, 5)])
+def test_verifier_roundings_against_independent_half_arithmetic(dtype, causal, window):
+    rng = np.random.default_rng(259 + 2 * int(causal) + window)
+    shape = (1, 2, 24, 16)
+    # values of full significand width, so p * v is inexact in the storage type almost everywhere; the second
+    # head has the reference's own input distribution, U[0, 10) (main.cu:69-70)
+    q, k, v = (rand_bits(rng, shape, dtype) for _ in range(3))
+    for x in (q, k, v):
+        x[0, 1] = ob.from_f32(rng.uniform(0.0, 10.0, size=shape[2:]).astype(np.float32), dtype)
+    scale = 1.0 / np.sqrt(shape[3])
+    want = independent_verifier(q, k, v, dtype, scale, causal, window)
+    # the check has teeth: without the product rounding, or without rounding p, other bits come out
+    lit = ob.literal(q, k, v, dtype, scale, causal, window, window)
+    o, _ = ob.full(q, k, v, dtype, scale, causal, window, window)
+    o_scalar, _ = ob.full(q, k, v, dtype, scale, causal, window, window, scalar=True)
+    assert np.array_equal(lit, want)
+    assert np.array_equal(o, want)
+    assert np.array_equal(o_scalar, want)
+
+
+def test_independent_half_arithmetic_is_sensitive_to_each_rounding():
+    """The independent literal itself: leaving out the p -> half rounding or the half product changes bits,
+    so agreement above cannot come from an insensitive input."""
+    rng = np.random.default_rng(7)
+    S, D = 24, 16
+    p = rng.uniform(0, 1, (S, S)).astype(np.float32)
+    p /= p.sum(1, keepdims=True)
+    v = rng.standard_normal((S, D)).astype(np.float16).astype(np.float32)
+
+    def pv(round_p, round_prod):
+        o = np.zeros((S, D), dtype=np.float32)
+        for c in range(S):
+            pc = _storage_round(p[:, c, None], F16) if round_p else p[:, c, None]
+            pr = pc * v[None, c, :]
+            o = o + (_storage_round(pr, F16) if round_prod else pr)
+        return ob.from_f32(o, F16)
+    base = pv(True, True)
+    assert not np.array_equal(base, pv(False, True))
+    assert not np.array_equal(base, pv(True, False))
+
+
 # ---------------------------------------------------------------- mask predicate, exhaustively
 @pytest.mark.parametrize("causal,wl,wr", [(False, -1, -1), (True, -1, -1), (False, 4, 4), (True, 9, -1), (False, 0, 3),
                                           (False, -1, 0), (False, 6, -1), (True, 0, -1)])
