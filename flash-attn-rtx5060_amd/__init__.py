@@ -44,7 +44,7 @@ FA_TILE_SKIP, FA_TILE_PARTIAL, FA_TILE_FULL = 0, 1, 2
 
 #: every symbol include/fa_fwd.h declares
 EXPORTED_SYMBOLS = (
-    "fa_fwd_validate", "fa_fwd", "run_flash_attention", "fa_strerror", "fa_last_device_error",
+    "fa_fwd_validate", "fa_fwd", "fa_init", "fa_reset_work_queues", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
@@ -72,6 +72,7 @@ class FaFwdParams(ctypes.Structure):
         ("q_strides", ctypes.c_longlong * 3), ("k_strides", ctypes.c_longlong * 3),
         ("v_strides", ctypes.c_longlong * 3), ("o_strides", ctypes.c_longlong * 3),
         ("S_kv", ctypes.c_int), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_ulonglong),
+        ("exact_first_rows", ctypes.c_int),
     ]
 
 
@@ -185,9 +186,10 @@ def host_lib():
 def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softmax_scale=None, causal=False,
                 window_left=-1, window_right=-1, dtype=FA_DTYPE_F16, sched=FA_SCHED_AUTO, alibi_ptr=0,
                 n_kv_heads=0, q_strides=None, k_strides=None, v_strides=None, o_strides=None, dropout_prob=0.0, seed=0,
-                S_kv=0, split_num=0, workspace_ptr=0, workspace_bytes=0):
+                S_kv=0, split_num=0, workspace_ptr=0, workspace_bytes=0, exact_first_rows=False):
     """A filled fa_fwd_params.  Strides are (batch, head, row) in elements, None = contiguous [B,N,S,d]."""
     p = FaFwdParams()
+    p.exact_first_rows = int(bool(exact_first_rows))
     p.alibi_slopes_ptr = alibi_ptr or None
     p.n_kv_heads = n_kv_heads
     p.dropout_prob, p.seed = dropout_prob, seed
@@ -203,16 +205,46 @@ def make_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, lse_ptr=0, softm
     return p
 
 
+def abi_strides(t):
+    """What the C ABI gets for a 4-d tensor [.., .., rows, d]: ``(tensor, strides)`` with strides None for a
+    dense tensor and the (batch, head, row) element strides otherwise.  The ABI reads an all-zero triple as
+    "dense", wants every stride to be a non-negative multiple of 8 elements, the row stride at least d and the
+    last dimension contiguous; a tensor that does not fit that (an expanded gradient with zero strides, an
+    odd slice) is replaced by a dense copy.  Strides of dimensions of size one carry no information and are
+    set to the dense value."""
+    if t.is_contiguous():
+        return t, None
+    st = list(t.stride())
+    shape = list(t.shape)
+    ok = st[3] == 1
+    dense = shape[3]
+    norm = [0, 0, 0]
+    for k in (2, 1, 0):
+        if shape[k] == 1:
+            norm[k] = max(dense, 8)
+        else:
+            norm[k] = st[k]
+            if st[k] <= 0 or st[k] % 8 != 0:
+                ok = False
+        dense *= shape[k]
+    if shape[2] > 1 and st[2] < shape[3]:
+        ok = False
+    if not ok:
+        return t.contiguous(), None
+    return t, tuple(norm)
+
+
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
                             return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None,
-                            dropout_prob=0.0, seed=0, splits=1):
+                            dropout_prob=0.0, seed=0, splits=1, exact_first_rows=False):
     """O, LSE = attention(q, k, v) on the GPU through fa_fwd().  q is [B, N, S, d], k and v are
     [B, Nk, S, d] with Nk dividing N (Nk < N: grouped-query attention); any strides with a contiguous last
     dimension are passed through (a [B, S, N, d] tensor is given as ``t.transpose(1, 2)``), any S >= 1.
     k and v may be longer or shorter than q ([B, Nk, S_kv, d]): query i then sits at key position
     i + S_kv - S.  ``splits``: an int > 1, or "auto", splits the keys of every query block over several
     workgroups and merges the partial results (few queries, long keys).
-    ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26)."""
+    ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26).
+    ``exact_first_rows``: see fa_fwd_params.exact_first_rows."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise ValueError("q, k, v must live on the GPU")
@@ -221,8 +253,7 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
     if q.dim() != 4 or k.shape != v.shape or k.dim() != 4 or (q.shape[0], q.shape[3]) != (
             k.shape[0], k.shape[3]) or k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0 or k.shape[2] == 0:
         raise ValueError("q must be [B, N, S, d], k and v [B, Nk, S_kv, d] with Nk dividing N")
-    if q.stride(3) != 1 or k.stride(3) != 1 or v.stride(3) != 1:
-        raise ValueError("the head dimension of q, k, v must be contiguous")
+    (q, q_st), (k, k_st), (v, v_st) = abi_strides(q), abi_strides(k), abi_strides(v)
     B, N, S, d = q.shape
     Nk, S_kv = k.shape[1], k.shape[2]
     if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
@@ -230,16 +261,19 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
         raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
     if out is None:
         out = torch.empty_like(q)          # keeps q's strides
-    if out.shape != q.shape or out.dtype != q.dtype or out.stride(3) != 1:
-        raise ValueError("out must have q's shape and dtype and a contiguous head dimension")
+    if out.shape != q.shape or out.dtype != q.dtype:
+        raise ValueError("out must have q's shape and dtype")
+    out_abi, o_st = abi_strides(out)
+    if out_abi is not out:
+        raise ValueError("out needs a contiguous head dimension and positive strides that are multiples of 8")
     if return_lse and lse is None:
         lse = torch.empty((B, N, S), dtype=torch.float32, device=q.device)
     p = make_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                     lse.data_ptr() if return_lse else 0, softmax_scale, causal, window_left, window_right,
                     FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16, sched,
                     0 if alibi_slopes is None else alibi_slopes.data_ptr(), 0 if Nk == N else Nk,
-                    *[None if t.is_contiguous() else tuple(t.stride()[:3]) for t in (q, k, v, out)],
-                    dropout_prob=dropout_prob, seed=seed, S_kv=0 if S_kv == S else S_kv)
+                    q_st, k_st, v_st, o_st,
+                    dropout_prob=dropout_prob, seed=seed, S_kv=0 if S_kv == S else S_kv, exact_first_rows=exact_first_rows)
     if splits == "auto":
         splits = lib().fa_fwd_suggest_splits(ctypes.byref(p))
     workspace = None
@@ -285,8 +319,8 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
     import torch
-    if not all(t.is_cuda and t.dtype == q.dtype and t.dim() == 4 and t.stride(3) == 1 for t in (q, k, v, o, do)):
-        raise ValueError("q, k, v, o, do must be 4-d GPU tensors of one dtype with a contiguous head dimension")
+    if not all(t.is_cuda and t.dtype == q.dtype and t.dim() == 4 for t in (q, k, v, o, do)):
+        raise ValueError("q, k, v, o, do must be 4-d GPU tensors of one dtype")
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise ValueError("tensors must be float16 or bfloat16")
     if o.shape != q.shape or do.shape != q.shape or k.shape != v.shape or (q.shape[0], q.shape[3]) != (
@@ -299,12 +333,19 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     if alibi_slopes is not None and not (alibi_slopes.is_cuda and alibi_slopes.dtype == torch.float32
                                          and alibi_slopes.is_contiguous() and tuple(alibi_slopes.shape) == (N,)):
         raise ValueError("alibi_slopes must be a contiguous float32 GPU tensor of shape [N]")
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)        # keep the inputs' strides
-    for t in (dq, dk, dv):
-        if t.stride(3) != 1:
-            raise ValueError("q, k, v must be laid out so that empty_like keeps a contiguous head dimension")
-    tensors = dict(q=q, k=k, v=v, o=o, do=do, dq=dq, dk=dk, dv=dv)
-    strides = {n: (None if t.is_contiguous() else tuple(t.stride()[:3])) for n, t in tensors.items()}
+    # inputs the ABI cannot address (zero strides of an expanded gradient, strides that are no multiple of 8)
+    # are replaced by dense copies; the gradients keep the strides of q, k, v where the ABI can write those
+    tensors, strides = {}, {}
+    for n, t in dict(q=q, k=k, v=v, o=o, do=do).items():
+        tensors[n], strides[n] = abi_strides(t)
+    q, k, v, o, do = (tensors[n] for n in ("q", "k", "v", "o", "do"))
+    for n, like in (("dq", q), ("dk", k), ("dv", v)):
+        g = torch.empty_like(like)                    # keeps a dense or permuted layout
+        g_abi, g_st = abi_strides(g)
+        if g_abi is not g:
+            g, g_st = torch.empty(like.shape, dtype=like.dtype, device=like.device), None
+        tensors[n], strides[n] = g, g_st
+    dq, dk, dv = tensors["dq"], tensors["dk"], tensors["dv"]
     p = make_bwd_params(B, N, S, d, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                         lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), softmax_scale, causal,
                         window_left, window_right, FA_DTYPE_BF16 if q.dtype == torch.bfloat16 else FA_DTYPE_F16,
@@ -334,7 +375,8 @@ def flash_attention(q, k, v, softmax_scale=None, causal=False, window_left=-1, w
         class _FlashAttention(torch.autograd.Function):
             @staticmethod
             def forward(ctx, q, k, v, opts):
-                o, lse = flash_attention_forward(q, k, v, **opts)
+                # exact products in every row: the logsumexp must be the one fa_bwd recomputes P from
+                o, lse = flash_attention_forward(q, k, v, exact_first_rows=True, **opts)
                 ctx.save_for_backward(q, k, v, o, lse)
                 ctx.opts = opts
                 return o
@@ -342,8 +384,6 @@ def flash_attention(q, k, v, softmax_scale=None, causal=False, window_left=-1, w
             @staticmethod
             def backward(ctx, do):
                 q, k, v, o, lse = ctx.saved_tensors
-                if do.stride(3) != 1:
-                    do = do.contiguous()
                 dq, dk, dv = flash_attention_backward(q, k, v, o, lse, do, **ctx.opts)
                 return dq, dk, dv, None
         _autograd_function = _FlashAttention

@@ -119,7 +119,7 @@ __device__ __forceinline__ void dma_4(const float *src, int index, uint32_t lds)
     const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
     const uint32_t voff = (uint32_t)index * 4u;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
 }
 
 __device__ __forceinline__ f32x16 zero16()
@@ -564,10 +564,16 @@ hipError_t launch_bwd(const FaBwdArgs &a, hipStream_t stream)
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512) + (DROPOUT ? kBwdWaves * 128 : 0);
     auto kq = fa_bwd_dq<BF16, D, MASKED, GENERAL, ALIBI, DROPOUT>;
     auto kkv = fa_bwd_dkdv<BF16, D, MASKED, GENERAL, ALIBI, DROPOUT>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kq), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
-    if (e != hipSuccess) return e;
+    // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
+    static std::atomic<unsigned long long> configured{0ull};
+    const unsigned long long dev_bit = 1ull << fa_launch_device();
+    if (!(configured.load(std::memory_order_relaxed) & dev_bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kq), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
+        if (e != hipSuccess) return e;
+        configured.fetch_or(dev_bit, std::memory_order_relaxed);
+    }
     hipLaunchKernelGGL(kq, dim3(grid_q), dim3(kBwdWaves * 64), smem_dq, stream, a);
     hipLaunchKernelGGL(kkv, dim3(grid_k), dim3(kBwdWaves * 64), smem_dkdv, stream, a);
     return hipGetLastError();

@@ -1,0 +1,21 @@
+// Per-device state of the library, set up once per device on the first call that needs it (or by fa_init):
+// the device address of the library's file-scope work-queue array and the CU count.  Everything after that
+// first call is a table lookup: no HIP query sits in the launch path.
+#ifndef FA_DEVICE_STATE_H
+#define FA_DEVICE_STATE_H
+#include <hip/hip_runtime.h>
+
+constexpr int kFaMaxDevices = 64;
+constexpr int kFaQueueSlots = 32;                              // work-queue counter sets per device
+
+struct FaDeviceState {
+    unsigned *queues;          // kFaQueueSlots sets of 16 words (nine used)
+    int compute_units;
+};
+
+// State of the current device (set up on first use).  Also records the device index for fa_launch_device().
+hipError_t fa_device_state(const FaDeviceState **state);
+// Index of the device the calling thread's current API call runs on (what fa_device_state saw last).
+int fa_launch_device();
+
+#endif

@@ -16,6 +16,7 @@
 #include "fa_fwd.h"
 #include "fa_bwd.h"
 #include "fa_bwd_args.h"
+#include "fa_device_state.h"
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
@@ -28,8 +29,6 @@ hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, hipStream_t stream);
 hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, hipStream_t stream);
-hipError_t fa_work_queue_base(unsigned **base);
-int fa_work_queue_slots();
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -47,28 +46,20 @@ int waves_for(int B, int N, int S)
 
 thread_local char g_last_error[256] = "";
 
-// device address of the work-queue array, per device (every device holds its own copy of the symbol)
-constexpr int kMaxDevices = 64;
-std::mutex g_queue_mutex;
-unsigned *g_queue_base[kMaxDevices] = {};
-std::atomic<unsigned> g_queue_ticket{0};
+std::atomic<unsigned> g_eager_ticket{0}, g_capture_ticket{0};
 
-hipError_t work_queue_for_launch(unsigned **queue)
+// A counter set for one FA_SCHED_QUEUE launch.  A launch that is being captured into a graph keeps its set for
+// every replay of that graph, so captured launches take their sets from the upper half of the table and eager
+// launches from the lower half: a replaying graph never shares counters with eager work on another stream.
+// Within a half the sets go round-robin.
+unsigned *work_queue_for_launch(const FaDeviceState *ds, hipStream_t stream)
 {
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-    {
-        std::lock_guard<std::mutex> lock(g_queue_mutex);
-        if (g_queue_base[dev] == nullptr) {
-            e = fa_work_queue_base(&g_queue_base[dev]);
-            if (e != hipSuccess) return e;
-        }
-    }
-    const unsigned slot = g_queue_ticket.fetch_add(1u) % (unsigned)fa_work_queue_slots();
-    *queue = g_queue_base[dev] + 16u * slot;
-    return hipSuccess;
+    constexpr unsigned half = (unsigned)kFaQueueSlots / 2u;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    const bool capturing = stream != nullptr && hipStreamIsCapturing(stream, &status) == hipSuccess &&
+                           status == hipStreamCaptureStatusActive;
+    const unsigned slot = capturing ? half + g_capture_ticket.fetch_add(1u) % half : g_eager_ticket.fetch_add(1u) % half;
+    return ds->queues + 16u * slot;
 }
 
 int device_fail(hipError_t e, const char *what)
@@ -239,7 +230,10 @@ int fa_fwd_suggest_splits(const fa_fwd_params *p)
     return n < 1 ? 1 : (int)n;
 }
 
-int fa_fwd_validate(const fa_fwd_params *p)
+namespace {
+int validate_layout(const fa_fwd_params *p);
+// everything but the workspace of a call with key splits
+int validate_no_workspace(const fa_fwd_params *p)
 {
     if (!p || !p->Q || !p->K || !p->V || !p->O) return FA_ERR_NULL_POINTER;
     if (p->B <= 0 || p->N <= 0 || p->S <= 0) return FA_ERR_BAD_SHAPE;
@@ -250,9 +244,24 @@ int fa_fwd_validate(const fa_fwd_params *p)
     const long long bh = (long long)p->B * p->N;
     if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
     if (p->S_kv < 0) return FA_ERR_BAD_SHAPE;
+    if ((long long)p->S + (p->S_kv > 0 ? p->S_kv : p->S) > 0x3fffffffLL) return FA_ERR_TOO_LARGE;   // tile and mask arithmetic is 32-bit
     if (base_items(p) * effective_splits(p) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    return validate_layout(p);
+}
+}  // namespace
+
+int fa_fwd_validate(const fa_fwd_params *p)
+{
+    const int st = validate_no_workspace(p);
+    if (st != FA_OK) return st;
     if (effective_splits(p) > 1 && (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
                                     p->workspace_bytes < fa_fwd_workspace_bytes(p))) return FA_ERR_WORKSPACE;
+    return FA_OK;
+}
+
+namespace {
+int validate_layout(const fa_fwd_params *p)
+{
     if (p->n_kv_heads < 0 || (p->n_kv_heads > 0 && p->N % p->n_kv_heads != 0)) return FA_ERR_LAYOUT;
     const void *ptrs[4] = {p->Q, p->K, p->V, p->O};
     const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
@@ -264,15 +273,15 @@ int fa_fwd_validate(const fa_fwd_params *p)
             if (st[k] < 0 || st[k] % 8 != 0) return FA_ERR_LAYOUT;
         if (st[2] < p->d) return FA_ERR_LAYOUT;
         if (st[2] > (1LL << 24)) return FA_ERR_TOO_LARGE;           // per-lane byte offsets inside a tile are 32-bit
+        // an output whose batch or head stride is zero would have several writers per element
+        if (t == 3 && ((p->B > 1 && st[0] == 0) || (p->N > 1 && st[1] == 0))) return FA_ERR_LAYOUT;
     }
     return FA_OK;
 }
 
-int fa_fwd(const fa_fwd_params *p, void *stream)
+// The forward pass with the partial results of key splits in `workspace` (ignored without splits).
+int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, void *stream)
 {
-    const int st = fa_fwd_validate(p);
-    if (st != FA_OK) return st;
-
     FaKernelArgs a;
     a.Q = static_cast<const uint16_t *>(p->Q);
     a.K = static_cast<const uint16_t *>(p->K);
@@ -288,7 +297,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.Sk = p->S_kv > 0 ? p->S_kv : p->S;
     a.n_splits = effective_splits(p);
     a.tiles_per_split = (key_tiles(p) + a.n_splits - 1) / a.n_splits;
-    a.o_part = static_cast<float *>(p->workspace);
+    a.o_part = static_cast<float *>(workspace);
     a.lse_part = a.o_part != nullptr ? a.o_part + (size_t)a.n_splits * p->B * p->N * p->S * p->d : nullptr;
     a.pack = packed_group(p);
     bool general = a.Hk != p->N || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
@@ -328,13 +337,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     // workgroups that walk the list themselves.
     long long grid = a.n_items;
     a.queue = nullptr;
-    int cus = kComputeUnits;
-    {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
-    }
-    const long long resident = (long long)cus * (waves == 8 ? 1 : 2);
+    const long long resident = (long long)ds->compute_units * (waves == 8 ? 1 : 2);
     // FA_SCHED_AUTO: with at most one item per resident workgroup there is nothing to schedule (and the
     // queue's counter round trips, 2.3 us each, would double the run time of a 7 us problem); with at most
     // two, the fixed snake pairs every long item with a short one; beyond that the work queue balances best.
@@ -344,10 +347,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         sched = a.n_items <= resident ? FA_SCHED_DISPATCH : a.n_items <= 2 * resident ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
     if (sched == FA_SCHED_PERSISTENT || sched == FA_SCHED_QUEUE) {
         if (grid > resident) grid = resident;
-        if (sched == FA_SCHED_QUEUE) {
-            hipError_t qe = work_queue_for_launch(&a.queue);
-            if (qe != hipSuccess) return device_fail(qe, "work queue");
-        }
+        if (sched == FA_SCHED_QUEUE) a.queue = work_queue_for_launch(ds, static_cast<hipStream_t>(stream));
     }
     const int shape = waves == 8 ? 0 : 1;
     // dropout: p in units of 1/256 (a key is kept iff its random byte is >= the threshold)
@@ -355,6 +355,7 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     a.drop_scale = 256.0f / (256.0f - (float)a.drop_threshold);
     a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
     a.seed_hi = (unsigned)(p->seed >> 32);
+    a.exact_first_rows = p->exact_first_rows != 0;
     hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
@@ -363,6 +364,35 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
         if (e != hipSuccess) return device_fail(e, "combine launch");
     }
     return FA_OK;
+}
+}  // namespace
+
+int fa_init(void)
+{
+    const FaDeviceState *ds = nullptr;
+    const hipError_t e = fa_device_state(&ds);
+    return e == hipSuccess ? FA_OK : device_fail(e, "device set-up");
+}
+
+int fa_fwd(const fa_fwd_params *p, void *stream)
+{
+    const int st = fa_fwd_validate(p);
+    if (st != FA_OK) return st;
+    const FaDeviceState *ds = nullptr;
+    const hipError_t e = fa_device_state(&ds);
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    return forward(p, p->workspace, ds, stream);
+}
+
+int fa_reset_work_queues(void)
+{
+    const FaDeviceState *ds = nullptr;
+    hipError_t e = fa_device_state(&ds);
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    e = hipDeviceSynchronize();
+    if (e != hipSuccess) return device_fail(e, "synchronize");
+    e = hipMemset(ds->queues, 0, (size_t)kFaQueueSlots * 16 * sizeof(unsigned));
+    return e == hipSuccess ? FA_OK : device_fail(e, "work queue reset");
 }
 
 int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, void *O, void *L, void *M,
@@ -469,6 +499,11 @@ int fa_bwd_validate(const fa_bwd_params *p)
             if (st[k] < 0 || st[k] % 8 != 0) return FA_ERR_LAYOUT;
         if (st[2] < p->d) return FA_ERR_LAYOUT;
         if (st[2] > (1LL << 24)) return FA_ERR_TOO_LARGE;           // per-lane byte offsets inside a tile are 32-bit
+        // a gradient whose batch or head stride is zero would have several writers per element
+        if (t >= 5) {
+            const int heads = t == 5 ? p->N : (p->n_kv_heads > 0 ? p->n_kv_heads : p->N);
+            if ((p->B > 1 && st[0] == 0) || (heads > 1 && st[1] == 0)) return FA_ERR_LAYOUT;
+        }
     }
     if (p->workspace == nullptr || reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0 ||
         p->workspace_bytes < fa_bwd_workspace_bytes(p)) return FA_ERR_WORKSPACE;
@@ -479,6 +514,11 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
 {
     const int st = fa_bwd_validate(p);
     if (st != FA_OK) return st;
+    {
+        const FaDeviceState *ds = nullptr;
+        const hipError_t de = fa_device_state(&ds);
+        if (de != hipSuccess) return device_fail(de, "device set-up");
+    }
     FaBwdArgs a;
     a.Q = static_cast<const uint16_t *>(p->Q);
     a.K = static_cast<const uint16_t *>(p->K);

@@ -2,17 +2,48 @@
 // 128 (the reference's only layout, src/main.cu:182), and the work-queue storage of the library.
 #include "fa_fwd_kernel_impl.h"
 
-// Work queues of FA_SCHED_QUEUE launches: kQueueSlots sets of nine counters, all zero between launches (the
-// last workgroup of a launch rewinds its set).  Launches take the sets round-robin, so launches that overlap
-// on one device do not share a set unless more than kQueueSlots of them are in flight at once.
-constexpr int kQueueSlots = 32;
-static __device__ __align__(256) unsigned g_work_queues[kQueueSlots][16];
+#include <atomic>
+#include <mutex>
 
-hipError_t fa_work_queue_base(unsigned **base)
+// Work queues of FA_SCHED_QUEUE launches: kFaQueueSlots sets of nine counters, all zero between launches (the
+// last workgroup of a launch rewinds its set).  Launches take the sets round-robin, so launches that overlap
+// on one device do not share a set unless more than half of kFaQueueSlots of them are in flight at once.
+static __device__ __align__(256) unsigned g_work_queues[kFaQueueSlots][16];
+
+namespace {
+std::mutex g_state_mutex;
+FaDeviceState g_state[kFaMaxDevices] = {};
+std::atomic<bool> g_state_ready[kFaMaxDevices] = {};
+thread_local int g_launch_device = 0;
+}  // namespace
+
+hipError_t fa_device_state(const FaDeviceState **state)
 {
-    return hipGetSymbolAddress(reinterpret_cast<void **>(base), HIP_SYMBOL(g_work_queues));
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kFaMaxDevices) return hipErrorInvalidDevice;
+    if (!g_state_ready[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_state_mutex);
+        if (!g_state_ready[dev].load(std::memory_order_relaxed)) {
+            // with `dev` current: each device holds its own copy of the arrays at its own address
+            FaDeviceState st = {};
+            e = hipGetSymbolAddress(reinterpret_cast<void **>(&st.queues), HIP_SYMBOL(g_work_queues));
+            if (e != hipSuccess) return e;
+            if (st.queues == nullptr) return hipErrorInvalidSymbol;
+            int n = 0;
+            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess) return e;
+            st.compute_units = n > 0 ? n : 256;
+            g_state[dev] = st;
+            g_state_ready[dev].store(true, std::memory_order_release);
+        }
+    }
+    g_launch_device = dev;
+    *state = &g_state[dev];
+    return hipSuccess;
 }
-int fa_work_queue_slots() { return kQueueSlots; }
+int fa_launch_device() { return g_launch_device; }
 
 hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                         hipStream_t stream)

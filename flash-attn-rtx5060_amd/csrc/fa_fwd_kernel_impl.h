@@ -42,6 +42,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
+#include "fa_device_state.h"
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
@@ -121,7 +124,7 @@ __device__ __forceinline__ void dma_16(const char *base, uint32_t voff, uint32_t
     const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
     const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
 }
 __device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -192,53 +195,74 @@ template <bool BF16> __device__ __forceinline__ float storage_product(float a, f
 template <bool BF16, int D>
 __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
                                     float *o32 /* null, or [rows][D] fp32 to write instead of Oh */,
-                                    float *lse_h, int S, int L, float scale, float slope,
+                                    float *lse_h, int rows /* queries 0..rows-1 */, int pos_off /* query i sits at key position i + pos_off */,
+                                    int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
                                     uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
-                                    float *sc /* LDS, 32*32 floats */)
+                                    float *sc /* LDS, 2*32*32 + 32 floats */)
 {
     constexpr int R = kFaithfulRows;
-    const int rows = S < R ? S : R;
+    float *ex = sc + R * R, *rsum = ex + R * R;
     const int tid = threadIdx.x, nthr = blockDim.x;
-    // scores (main.cu:189-197), masked entries -inf (main.cu:210-229)
+    // scores (main.cu:189-197), masked entries -inf (main.cu:210-229); query i at position p sees keys p-L..p
     for (int idx = tid; idx < R * R; idx += nthr) {
-        const int i = idx / R, j = idx % R;
+        const int i = idx / R, j = idx % R, p = i + pos_off;
         float s = -INFINITY;
-        if (i < rows && j <= i && i - j <= L) {
+        if (i < rows && j <= p && p - j <= L) {
             float sum = 0.0f;
             for (int t = 0; t < D; ++t)
                 sum += storage_product<BF16>(storage_to_f32<BF16>(Qh[(size_t)i * q_rs + t]), storage_to_f32<BF16>(Kh[(size_t)j * k_rs + t]));
             s = sum * scale;
             // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
-            if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(i - j)));
+            if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(p - j)));
         }
         sc[idx] = s;
     }
     __syncthreads();
-    // softmax of each row (main.cu:232-252), p rounded to the storage type (main.cu:259)
-    if (tid < rows) {
-        float *row = sc + tid * R;
+    // softmax of each row (main.cu:232-252).  The row maximum does not depend on the order it is taken in and
+    // the exponentials are independent, so every thread does one element; only the row sum has to add in
+    // index order, and one thread per row does that.
+    for (int idx = tid; idx < R * R; idx += nthr) {
+        const int i = idx / R;
+        const float *row = sc + i * R;
         float mx = -INFINITY;
-        for (int j = 0; j <= tid; ++j) mx = fmaxf(mx, row[j]);
+        for (int j = 0; j < R; ++j) mx = fmaxf(mx, row[j]);
+        ex[idx] = (i < rows && sc[idx] != -INFINITY) ? expf(sc[idx] - mx) : 0.0f;
+    }
+    __syncthreads();
+    if (tid < rows) {
+        const float *row = ex + tid * R;
         float sum = 0.0f;
-        for (int j = 0; j <= tid; ++j) { row[j] = expf(row[j] - mx); sum += row[j]; }
-        for (int j = 0; j <= tid; ++j) {
-            float pj = row[j] / sum;
+        for (int j = 0; j < R; ++j) sum += row[j];          // masked entries are +0: they change no bit of the sum
+        rsum[tid] = sum;
+        if (lse_h != nullptr) {
+            float mx = -INFINITY;
+            for (int j = 0; j < R; ++j) mx = fmaxf(mx, sc[tid * R + j]);
+            lse_h[tid] = mx + logf(sum);
+        }
+    }
+    __syncthreads();
+    // p rounded to the storage type (main.cu:259)
+    for (int idx = tid; idx < R * R; idx += nthr) {
+        const int i = idx / R, j = idx % R;
+        float pj = 0.0f;
+        if (i < rows && sc[idx] != -INFINITY) {
+            pj = ex[idx] / rsum[i];
             if (drop_threshold != 0u) {        // keys 0..31: one 32-key block, two Philox blocks per query
-                const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)tid, (uint32_t)((j >> 2) & 1));
+                const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)(i + pos_off), (uint32_t)((j >> 2) & 1));
                 pj = dropout_keep_byte(d, 4 * (j >> 3) + (j & 3), drop_threshold) ? __fmul_rn(pj, drop_scale) : 0.0f;
             }
-            row[j] = storage_to_f32<BF16>(f32_to_storage<BF16>(pj));
+            pj = storage_to_f32<BF16>(f32_to_storage<BF16>(pj));
         }
-        if (lse_h != nullptr) lse_h[tid] = mx + logf(sum);
+        ex[idx] = pj;
     }
     __syncthreads();
     // weighted sum (main.cu:255-263), keys in ascending order; masked keys have p = 0 and add nothing
     for (int idx = tid; idx < rows * D; idx += nthr) {
-        const int i = idx / D, t = idx % D;
-        const int lo = i - L > 0 ? i - L : 0;
+        const int i = idx / D, t = idx % D, p = i + pos_off;
+        const int lo = p - L > 0 ? p - L : 0;
         float sum = 0.0f;
-        for (int j = lo; j <= i; ++j) sum += storage_product<BF16>(sc[i * R + j], storage_to_f32<BF16>(Vh[(size_t)j * v_rs + t]));
+        for (int j = lo; j <= p; ++j) sum += storage_product<BF16>(ex[i * R + j], storage_to_f32<BF16>(Vh[(size_t)j * v_rs + t]));
         if (o32 != nullptr) o32[(size_t)i * D + t] = storage_to_f32<BF16>(f32_to_storage<BF16>(sum));
         else Oh[(size_t)i * o_rs + t] = f32_to_storage<BF16>(sum);
     }
@@ -793,7 +817,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
-    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off == 0 && split == 0 && pack == 1;
+    // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32;
+    // fa_fwd_params.exact_first_rows switches the path off)
+    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
+    const int f_rows = !faithful ? 0 : !GENERAL ? kFaithfulRows : (kFaithfulRows - pos_off < S ? kFaithfulRows - pos_off : S);
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
     // own keys), which fa_combine_splits merges.
     float *o_part = nullptr, *lse_part = nullptr;
@@ -806,11 +833,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides)
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
-            if (faithful && wave == 0 && b == 0) continue;
+            if (!GENERAL && faithful && wave == 0 && b == 0) continue;
             // the row's index in its head's [S, ...] output, counted from head `bh` (packed groups: row_head
             // heads further on; their logsumexp and partial rows follow at S per head, their O rows at o_hs)
             const int q = GENERAL ? row_head[b] * S + row_pos[b] : my_q + 32 * b;
             if (!row_ok[b]) continue;              // a row past the end
+            if (GENERAL && b == 0 && my_q < f_rows) continue;      // written by faithful_first_rows below
             const float l_half = l_a[b] + l_b[b];
             const float l_tot = l_half + swap_halves(l_half);
             const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
@@ -844,7 +872,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     }
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
-                                     S, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
+                                     f_rows, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
                                      a.seed_lo, a.seed_hi, (uint32_t)bh, reinterpret_cast<float *>(smem));
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
@@ -899,8 +927,14 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
     constexpr int TILEB = kBlockKeys * D * 2;
     const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
     auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
+    // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
+    static std::atomic<unsigned long long> configured{0ull};
+    const unsigned long long dev_bit = 1ull << fa_launch_device();
+    if (!(configured.load(std::memory_order_relaxed) & dev_bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+        configured.fetch_or(dev_bit, std::memory_order_relaxed);
+    }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
     return hipGetLastError();
 }

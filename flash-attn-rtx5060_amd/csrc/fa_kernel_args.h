@@ -40,6 +40,8 @@ struct FaKernelArgs {
     unsigned drop_threshold;   // key kept iff its byte >= threshold; p = threshold / 256
     float drop_scale;          // 256 / (256 - threshold)
     unsigned seed_lo, seed_hi;
+    // --- masked instantiations
+    int exact_first_rows;      // 1: no row is recomputed in the reference verifier's rounded-product arithmetic
 };
 
 #endif

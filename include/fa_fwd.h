@@ -106,6 +106,14 @@ typedef struct fa_fwd_params {
                                  key get O = 0 and L = -inf                                              */
     void *workspace;          /* device scratch for split_num > 1, at least fa_fwd_workspace_bytes()    */
     unsigned long long workspace_bytes;
+    int exact_first_rows;     /* 0 (default): under a causal-type mask (no key right of the query) the query
+                                 rows that see at most 32 keys are computed in the arithmetic of the
+                                 reference's CPU verifier, every q*k and p*v product rounded to the storage
+                                 type (main.cu:193,259): there an output can be as large as the values
+                                 themselves and the verifier's own rounding, up to 3e-3 at unit variance, is
+                                 larger than the tolerance a drop-in has to meet against it.  1: those rows
+                                 use exact products and fp32 accumulation like every other row, and their
+                                 logsumexp is the one a backward pass recomputes P from (fa_bwd)          */
 } fa_fwd_params;
 
 /* Checks a parameter block without touching any device.  Returns FA_OK or the
@@ -118,11 +126,25 @@ unsigned long long fa_fwd_workspace_bytes(const fa_fwd_params *p);
 /* A split count that fills the device for these shapes (1 when the problem has enough work items anyway). */
 int fa_fwd_suggest_splits(const fa_fwd_params *p);
 
+/* Optional: sets up the library's state for the current device (looks up the address of its
+ * file-scope work-queue array and the CU count) so that the first fa_fwd call does not.  Every entry point that
+ * needs the state does the same on its first call on a device. */
+int fa_init(void);
+
 /* Enqueues the forward pass on `stream` and returns without synchronising.
  * Allocates nothing; Q/K/V are read-only, O (and L when non-NULL) are
  * overwritten.  Re-entrant: the library keeps no per-call global state
  * (the reference keeps four global CUtensorMaps, flash_forward.h:17-20). */
 int fa_fwd(const fa_fwd_params *p, void *stream);
+
+/* FA_SCHED_QUEUE keeps per-launch counters in the library's own device memory (32 sets per device, eager
+ * launches rotate through 16 of them, launches captured into graphs through the other 16); the last workgroup
+ * of a launch rewinds its set.  Restrictions: more than 16 queue launches in flight at once on one device
+ * share a set and give wrong results, as do two graphs captured more than 16 launches apart that replay
+ * concurrently; use FA_SCHED_PERSISTENT or FA_SCHED_DISPATCH for such callers.  A launch that was killed
+ * half-way (device reset, process signal) leaves its set dirty: fa_reset_work_queues() waits for the device
+ * and zeroes all sets of the current device.  Never call it while launches are being captured. */
+int fa_reset_work_queues(void);
 
 /*
  * The reference's entry point, same name, argument order and meaning

@@ -153,9 +153,53 @@ def test_validate_status_codes(fa):
     assert status(v_strides=(-8, 64, 512)) == fa.FA_ERR_LAYOUT
     assert status(o_strides=(0, 0, 1 << 25)) == fa.FA_ERR_TOO_LARGE
     assert status(q_ptr=0x1008) == fa.FA_ERR_LAYOUT
+    # an output with a zero batch or head stride would have several writers per element; inputs may broadcast
+    assert status(o_strides=(0, 2048 * 64, 64)) == fa.FA_ERR_LAYOUT
+    assert status(o_strides=(8 * 2048 * 64, 0, 64)) == fa.FA_ERR_LAYOUT
+    assert status(k_strides=(0, 2048 * 64, 64)) == fa.FA_OK
+    assert status(B=1, o_strides=(0, 2048 * 64, 64)) == fa.FA_OK
+    # tile and mask arithmetic is 32-bit: S + S_kv must stay below 2^30
+    assert status(B=1, N=1, S=0x20000000) == fa.FA_ERR_TOO_LARGE
+    assert status(B=1, N=1, S=128, S_kv=0x3fffff80) == fa.FA_ERR_TOO_LARGE
+    assert status(B=1, N=1, S=128, S_kv=0x3fffff00) == fa.FA_OK
     # fa_fwd itself refuses the same blocks before touching any device
     p = fa.make_params(**dict(ok, d=96))
     assert L.fa_fwd(ctypes.byref(p), None) == fa.FA_ERR_HEAD_DIM
+
+
+def test_python_stride_marshalling():
+    """What the binding hands the ABI for tensors whose strides the ABI cannot take as they are."""
+    import torch
+    fa = __import__("conftest").load_package()
+    dense = torch.zeros(2, 4, 16, 64, dtype=torch.float16)
+    assert fa.abi_strides(dense) == (dense, None) or fa.abi_strides(dense)[1] is None
+    bshd = torch.zeros(2, 16, 4, 64, dtype=torch.float16).transpose(1, 2)
+    t, st = fa.abi_strides(bshd)
+    assert t is bshd and st == (16 * 4 * 64, 64, 4 * 64)
+    # an expanded gradient (zero strides, as produced by o.sum().backward()) must not reach the ABI as
+    # (0, 0, 0), which means "dense": it is copied
+    expanded = torch.ones(64, dtype=torch.float16).expand(2, 4, 16, 64)
+    assert expanded.stride() == (0, 0, 0, 1)
+    t, st = fa.abi_strides(expanded)
+    assert st is None and t.is_contiguous() and t.shape == expanded.shape
+    part = torch.zeros(2, 1, 16, 64, dtype=torch.float16).expand(2, 4, 16, 64)       # one zero stride
+    t, st = fa.abi_strides(part)
+    assert st is None and t.is_contiguous()
+    # strides that are no multiple of 8 elements, or a head dimension that is not contiguous: copied
+    odd = torch.zeros(2, 4, 16, 68, dtype=torch.float16)[..., :64]
+    t, st = fa.abi_strides(odd)
+    assert st is None and t.is_contiguous()
+    strided_d = torch.zeros(2, 4, 16, 128, dtype=torch.float16)[..., ::2]
+    t, st = fa.abi_strides(strided_d)
+    assert st is None and t.is_contiguous()
+    # a row stride larger than d that is a multiple of 8 passes through
+    wide = torch.zeros(2, 4, 16, 96, dtype=torch.float16)[..., :64]
+    t, st = fa.abi_strides(wide)
+    assert t is wide and st == (4 * 16 * 96, 16 * 96, 96)
+    # strides of size-one dimensions carry no information and never make the triple all zero or odd
+    one = torch.zeros(1, 4, 16, 96, dtype=torch.float16)[..., :64].as_strided((1, 4, 16, 64), (3, 16 * 96, 96, 1))
+    t, st = fa.abi_strides(one)
+    assert t is one and st[1:] == (16 * 96, 96) and st[0] % 8 == 0 and st[0] > 0
 
 
 def test_reference_entry_point_rejects_unsupported_flags(fa):
