@@ -817,9 +817,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
-    // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32;
+    // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32
+    // (with more queries than keys, pos_off < 0, the path is not taken);
     // fa_fwd_params.exact_first_rows switches the path off)
-    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
+    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off >= 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
     const int f_rows = !faithful ? 0 : !GENERAL ? kFaithfulRows : (kFaithfulRows - pos_off < S ? kFaithfulRows - pos_off : S);
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
     // own keys), which fa_combine_splits merges.

@@ -82,8 +82,12 @@ def test_random_configurations(fa):
         o_ref, lse_ref, dq_ref, dk_ref, dv_ref = reference(q, k, v, do, causal, wl, wr, slopes, keep)
         half = dtype == torch.float16
         assert bool(torch.isfinite(o.float()).all()), what
+        # the tolerance, or one ulp of the storage type where a row of few keys makes the output so large
+        # (|O| >= 4) that one ulp exceeds it: p and the result are each rounded once to the storage type
         # (an indexing mistake shows up as an error of order one)
-        assert float((o.float() - o_ref).abs().max()) <= (2e-3 if half else 1.6e-2) * grow, what
+        one_ulp = torch.exp2(torch.floor(torch.log2(o_ref.abs().clamp_min(1e-4))) - (10 if half else 7))
+        bound = torch.maximum(one_ulp, torch.full_like(one_ulp, 2e-3 if half else 1.6e-2)) * grow
+        assert bool(((o.float() - o_ref).abs() <= bound).all()), (what, float((o.float() - o_ref).abs().max()))
         seen = torch.isfinite(lse_ref)
         assert bool((lse[~seen] == float("-inf")).all()), what
         if bool(seen.any()):
