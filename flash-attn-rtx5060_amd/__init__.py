@@ -37,6 +37,7 @@ FA_ERR_NO_DEVICE = -9
 FA_ERR_TOO_LARGE = -10
 FA_ERR_LAYOUT = -11
 FA_ERR_WORKSPACE = -12
+FA_ERR_SCRATCH_LIMIT = -13
 FA_DTYPE_F16 = 0
 FA_DTYPE_BF16 = 1
 FA_SCHED_AUTO, FA_SCHED_DISPATCH, FA_SCHED_PERSISTENT, FA_SCHED_QUEUE = 0, 1, 2, 3
@@ -44,7 +45,8 @@ FA_TILE_SKIP, FA_TILE_PARTIAL, FA_TILE_FULL = 0, 1, 2
 
 #: every symbol include/fa_fwd.h declares
 EXPORTED_SYMBOLS = (
-    "fa_fwd_validate", "fa_fwd", "fa_init", "fa_reset_work_queues", "run_flash_attention", "fa_strerror", "fa_last_device_error",
+    "fa_fwd_validate", "fa_fwd", "fa_init", "fa_fwd_split_static", "fa_fwd_static_scratch_bytes",
+    "fa_reset_work_queues", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
@@ -126,6 +128,8 @@ def lib():
         L.fa_last_device_error.restype = ctypes.c_char_p
         L.fa_fwd_validate.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.fa_fwd.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
+        L.fa_fwd_split_static.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
+        L.fa_fwd_static_scratch_bytes.restype = ctypes.c_ulonglong
         L.fa_fwd_workspace_bytes.restype = ctypes.c_ulonglong
         L.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.fa_fwd_suggest_splits.argtypes = [ctypes.POINTER(FaFwdParams)]
@@ -236,7 +240,7 @@ def abi_strides(t):
 
 def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
                             return_lse=True, out=None, lse=None, sched=FA_SCHED_AUTO, alibi_slopes=None,
-                            dropout_prob=0.0, seed=0, splits=1, exact_first_rows=False):
+                            dropout_prob=0.0, seed=0, splits=1, exact_first_rows=False, static_scratch=False):
     """O, LSE = attention(q, k, v) on the GPU through fa_fwd().  q is [B, N, S, d], k and v are
     [B, Nk, S, d] with Nk dividing N (Nk < N: grouped-query attention); any strides with a contiguous last
     dimension are passed through (a [B, S, N, d] tensor is given as ``t.transpose(1, 2)``), any S >= 1.
@@ -244,7 +248,8 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
     i + S_kv - S.  ``splits``: an int > 1, or "auto", splits the keys of every query block over several
     workgroups and merges the partial results (few queries, long keys).
     ``alibi_slopes``: fp32 GPU tensor [N]; slope[h]*|i-j| is subtracted from every scaled score (mask.h:21-26).
-    ``exact_first_rows``: see fa_fwd_params.exact_first_rows."""
+    ``exact_first_rows``: see fa_fwd_params.exact_first_rows.  ``static_scratch``: go through
+    fa_fwd_split_static (the key splits' partial results in the library's own static device array)."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise ValueError("q, k, v must live on the GPU")
@@ -280,11 +285,12 @@ def flash_attention_forward(q, k, v, softmax_scale=None, causal=False, window_le
     if splits and splits > 1:
         p.split_num = int(splits)
         need = lib().fa_fwd_workspace_bytes(ctypes.byref(p))
-        if need:
+        if need and not static_scratch:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)   # stream-ordered: freed after the launch
             p.workspace, p.workspace_bytes = workspace.data_ptr(), need
     stream = torch.cuda.current_stream(q.device).cuda_stream
-    st = lib().fa_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
+    entry = lib().fa_fwd_split_static if static_scratch else lib().fa_fwd
+    st = entry(ctypes.byref(p), ctypes.c_void_p(stream))
     if st != FA_OK:
         raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
     return (out, lse) if return_lse else out

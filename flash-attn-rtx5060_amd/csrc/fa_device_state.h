@@ -1,5 +1,5 @@
 // Per-device state of the library, set up once per device on the first call that needs it (or by fa_init):
-// the device address of the library's file-scope work-queue array and the CU count.  Everything after that
+// the device addresses of the library's two file-scope device arrays and the CU count.  Everything after that
 // first call is a table lookup: no HIP query sits in the launch path.
 #ifndef FA_DEVICE_STATE_H
 #define FA_DEVICE_STATE_H
@@ -7,9 +7,11 @@
 
 constexpr int kFaMaxDevices = 64;
 constexpr int kFaQueueSlots = 32;                              // work-queue counter sets per device
+constexpr unsigned long long kFaStaticScratchBytes = 32ull << 20;   // key-split scratch per device
 
 struct FaDeviceState {
     unsigned *queues;          // kFaQueueSlots sets of 16 words (nine used)
+    unsigned char *scratch;    // kFaStaticScratchBytes bytes, 256-byte aligned
     int compute_units;
 };
 

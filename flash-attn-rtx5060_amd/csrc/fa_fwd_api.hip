@@ -87,6 +87,7 @@ const char *fa_strerror(int status)
     case FA_ERR_DEVICE: return "HIP runtime error";
     case FA_ERR_NO_DEVICE: return "no gfx950 device visible";
     case FA_ERR_TOO_LARGE: return "problem too large for the kernel's index range";
+    case FA_ERR_SCRATCH_LIMIT: return "the partial results of this call exceed the library's static scratch (fa_fwd_static_scratch_bytes): use fewer splits or fa_fwd with a workspace";
     default: return "unknown status";
     }
 }
@@ -382,6 +383,20 @@ int fa_fwd(const fa_fwd_params *p, void *stream)
     const hipError_t e = fa_device_state(&ds);
     if (e != hipSuccess) return device_fail(e, "device set-up");
     return forward(p, p->workspace, ds, stream);
+}
+
+unsigned long long fa_fwd_static_scratch_bytes(void) { return kFaStaticScratchBytes; }
+
+int fa_fwd_split_static(const fa_fwd_params *p, void *stream)
+{
+    const int st = validate_no_workspace(p);
+    if (st != FA_OK) return st;
+    if (fa_fwd_workspace_bytes(p) > kFaStaticScratchBytes) return FA_ERR_SCRATCH_LIMIT;
+    const FaDeviceState *ds = nullptr;
+    const hipError_t e = fa_device_state(&ds);      // first call on a device: looks the two arrays up, no allocation
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    // the kernels get the array's device address, exactly as they get a caller's workspace in fa_fwd
+    return forward(p, ds->scratch, ds, stream);
 }
 
 int fa_reset_work_queues(void)

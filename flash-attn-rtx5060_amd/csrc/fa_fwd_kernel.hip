@@ -10,6 +10,11 @@
 // on one device do not share a set unless more than half of kFaQueueSlots of them are in flight at once.
 static __device__ __align__(256) unsigned g_work_queues[kFaQueueSlots][16];
 
+// Scratch of fa_fwd_split_static: the fp32 partial outputs and logsumexps of a launch with key splits, for
+// callers that may not allocate a workspace.  Every device holds its own copy for the life of the process.
+// In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
+static __device__ __align__(256) unsigned char g_split_scratch[kFaStaticScratchBytes];
+
 namespace {
 std::mutex g_state_mutex;
 FaDeviceState g_state[kFaMaxDevices] = {};
@@ -30,7 +35,9 @@ hipError_t fa_device_state(const FaDeviceState **state)
             FaDeviceState st = {};
             e = hipGetSymbolAddress(reinterpret_cast<void **>(&st.queues), HIP_SYMBOL(g_work_queues));
             if (e != hipSuccess) return e;
-            if (st.queues == nullptr) return hipErrorInvalidSymbol;
+            e = hipGetSymbolAddress(reinterpret_cast<void **>(&st.scratch), HIP_SYMBOL(g_split_scratch));
+            if (e != hipSuccess) return e;
+            if (st.queues == nullptr || st.scratch == nullptr) return hipErrorInvalidSymbol;
             int n = 0;
             e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
             if (e != hipSuccess) return e;

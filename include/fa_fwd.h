@@ -38,7 +38,8 @@ enum {
     FA_ERR_TOO_LARGE = -10,        /* B*N*S*d or the work-item count overflows the kernel's index range */
     FA_ERR_LAYOUT = -11,           /* a stride is not a multiple of 8 elements or too small, n_kv_heads does
                                       not divide N, or a tensor pointer is not 16-byte aligned */
-    FA_ERR_WORKSPACE = -12         /* split_num > 1 and the workspace is NULL, misaligned or too small */
+    FA_ERR_WORKSPACE = -12,        /* split_num > 1 and the workspace is NULL, misaligned or too small */
+    FA_ERR_SCRATCH_LIMIT = -13     /* fa_fwd_split_static: the partial results do not fit the static scratch */
 };
 
 enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
@@ -126,8 +127,8 @@ unsigned long long fa_fwd_workspace_bytes(const fa_fwd_params *p);
 /* A split count that fills the device for these shapes (1 when the problem has enough work items anyway). */
 int fa_fwd_suggest_splits(const fa_fwd_params *p);
 
-/* Optional: sets up the library's state for the current device (looks up the address of its
- * file-scope work-queue array and the CU count) so that the first fa_fwd call does not.  Every entry point that
+/* Optional: sets up the library's state for the current device (looks up the addresses of its two
+ * file-scope device arrays and the CU count) so that the first fa_fwd call does not.  Every entry point that
  * needs the state does the same on its first call on a device. */
 int fa_init(void);
 
@@ -136,6 +137,21 @@ int fa_init(void);
  * overwritten.  Re-entrant: the library keeps no per-call global state
  * (the reference keeps four global CUtensorMaps, flash_forward.h:17-20). */
 int fa_fwd(const fa_fwd_params *p, void *stream);
+
+/*
+ * fa_fwd for callers that cannot allocate device memory.  No counterpart in the reference (which has no
+ * key splits at all); it exists for callers under HIP graph capture, in tight serving loops or in harnesses
+ * that forbid hipMalloc, who cannot provide the workspace a call with split_num > 1 needs.  Same arguments,
+ * results and kernels as fa_fwd; `workspace` and `workspace_bytes` are ignored and the fp32 partial results
+ * of the key splits go to a file-scope device array of fa_fwd_static_scratch_bytes() = 32 MiB that every
+ * device holds for the life of the process.  Calls no allocating routine.  Returns FA_ERR_SCRATCH_LIMIT when
+ * fa_fwd_workspace_bytes(p) exceeds that size.  All calls on one device share the array: two such calls that
+ * overlap in time on one device (different streams, or a graph replay next to eager work) race; calls
+ * ordered on one stream do not.  Nothing in the array has to start at zero: every partial row the merge
+ * kernel reads is written by the launch before it.
+ */
+int fa_fwd_split_static(const fa_fwd_params *p, void *stream);
+unsigned long long fa_fwd_static_scratch_bytes(void);
 
 /* FA_SCHED_QUEUE keeps per-launch counters in the library's own device memory (32 sets per device, eager
  * launches rotate through 16 of them, launches captured into graphs through the other 16); the last workgroup

@@ -167,6 +167,21 @@ def test_validate_status_codes(fa):
     assert L.fa_fwd(ctypes.byref(p), None) == fa.FA_ERR_HEAD_DIM
 
 
+def test_static_scratch_entry_point_checks_before_touching_a_device(fa):
+    L = fa.lib()
+    limit = L.fa_fwd_static_scratch_bytes()
+    assert limit == 32 << 20
+    ok = dict(B=2, N=8, S=4, d=64, q_ptr=0x1000, k_ptr=0x2000, v_ptr=0x3000, o_ptr=0x4000, S_kv=4096)
+    # the same argument checks as fa_fwd, workspace fields ignored
+    assert L.fa_fwd_split_static(ctypes.byref(fa.make_params(**dict(ok, d=96))), None) == fa.FA_ERR_HEAD_DIM
+    assert L.fa_fwd_split_static(None, None) == fa.FA_ERR_NULL_POINTER
+    # partial results beyond the static array are refused with a status of their own
+    big = fa.make_params(**dict(ok, B=8, N=32, S=128, S_kv=8192, d=128, split_num=16))
+    assert L.fa_fwd_workspace_bytes(ctypes.byref(big)) > limit
+    assert L.fa_fwd_split_static(ctypes.byref(big), None) == fa.FA_ERR_SCRATCH_LIMIT
+    assert b"static scratch" in L.fa_strerror(fa.FA_ERR_SCRATCH_LIMIT)
+
+
 def test_python_stride_marshalling():
     """What the binding hands the ABI for tensors whose strides the ABI cannot take as they are."""
     import torch
