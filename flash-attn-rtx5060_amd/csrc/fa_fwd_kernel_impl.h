@@ -130,6 +130,18 @@ __device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcn
 
 template <int V> struct IntC { static constexpr int value = V; };
 
+// Per-item timeline for performance work: compiled only with -DFA_TIMELINE (never in the shipped library).
+// Thread 0 of every workgroup writes sixteen 64-bit words per work item: item, XCD and CU id, then the 100 MHz
+// wall clock when the item was taken, after the prologue, after the tile loop, after the epilogue, after
+// the first-rows path, the numbers of fill+drain and steady iterations, the tile range, and (words 10-14) the
+// shader clock counter at the same five points.
+#ifdef FA_TIMELINE
+__device__ long long *g_fa_timeline = nullptr;
+#define FA_TL(slot) do { if (tl != nullptr) { tl[slot] = (long long)__builtin_amdgcn_s_memrealtime(); tl[slot + 8] = (long long)__builtin_amdgcn_s_memtime(); } } while (0)
+#else
+#define FA_TL(slot) do { } while (0)
+#endif
+
 // ---------------------------------------------------------------------------
 // First rows of a causal head, in the reference's own arithmetic.
 //
@@ -186,12 +198,30 @@ template <bool BF16> __device__ __forceinline__ uint16_t f32_to_storage(float x)
     if (BF16) return __builtin_bit_cast(uint16_t, (__bf16)x);
     return __builtin_bit_cast(uint16_t, (_Float16)x);
 }
-// storage-type product of two storage-type values: the fp32 product is exact, one rounding to nearest even
-template <bool BF16> __device__ __forceinline__ float storage_product(float a, float b)
+// Two storage-type products a.lo * b.lo and a.hi * b.hi of packed storage-type values, each rounded once to the
+// storage type (round to nearest even) and widened to fp32: the reference's half x half -> half product
+// (main.cu:193,259).  fp16: v_pk_mul_f16 rounds exactly so; the empty asm keeps the compiler from contracting
+// the product with the addition that follows into one fused operation, which would skip the rounding.
+// bf16: the fp32 product of two bf16 values is exact, then one rounding.
+template <bool BF16> __device__ __forceinline__ f32x2 storage_product2(uint32_t a, uint32_t b)
 {
-    return storage_to_f32<BF16>(f32_to_storage<BF16>(a * b));
+    if (!BF16) {
+        f16x2 pr = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
+        uint32_t bits = __builtin_bit_cast(uint32_t, pr);
+        asm volatile("" : "+v"(bits));
+        pr = __builtin_bit_cast(f16x2, bits);
+        return f32x2{(float)pr[0], (float)pr[1]};
+    }
+    const f32x2 exact = {__builtin_bit_cast(float, a << 16) * __builtin_bit_cast(float, b << 16),
+                         __builtin_bit_cast(float, a & 0xffff0000u) * __builtin_bit_cast(float, b & 0xffff0000u)};
+    const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(exact, bf16x2));
+    return f32x2{__builtin_bit_cast(float, r << 16), __builtin_bit_cast(float, r & 0xffff0000u)};
 }
 
+// Queries 0..rows-1 of a head (query i at key position i + pos_off, all positions below 32) against keys
+// 0..31.  The 32 x D blocks of Q, K and V are staged in LDS once (K with its 16-byte chunks XOR-swizzled by the
+// row, so that 32 lanes reading one chunk of 32 different rows do not collide), everything else runs from
+// there.  LDS use: 3 * 32 * D * 2 + 2 * 4096 + 128 bytes.
 template <bool BF16, int D>
 __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
                                     float *o32 /* null, or [rows][D] fp32 to write instead of Oh */,
@@ -199,19 +229,43 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
                                     int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
                                     uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
-                                    float *sc /* LDS, 2*32*32 + 32 floats */)
+                                    char *lds)
 {
-    constexpr int R = kFaithfulRows;
-    float *ex = sc + R * R, *rsum = ex + R * R;
+    constexpr int R = kFaithfulRows, CPR = D / 8;
+    uint16_t *Qs = reinterpret_cast<uint16_t *>(lds), *Ks = Qs + R * D, *Vs = Ks + R * D;
+    float *sc = reinterpret_cast<float *>(Vs + R * D), *ex = sc + R * R, *rsum = ex + R * R;
+    uint32_t *pbits = reinterpret_cast<uint32_t *>(ex);     // after the softmax: p as two copies of its storage bits
     const int tid = threadIdx.x, nthr = blockDim.x;
+    const int nkeys = rows + pos_off;                       // keys 0..nkeys-1 are the ones any of these queries sees
+    for (int idx = tid; idx < R * CPR; idx += nthr) {
+        const int row = idx / CPR, c = idx % CPR;
+        u32x4 q4 = {0, 0, 0, 0}, k4 = {0, 0, 0, 0}, v4 = {0, 0, 0, 0};
+        if (row < rows) q4 = *reinterpret_cast<const u32x4 *>(Qh + (size_t)row * q_rs + 8 * c);
+        if (row < nkeys) {
+            k4 = *reinterpret_cast<const u32x4 *>(Kh + (size_t)row * k_rs + 8 * c);
+            v4 = *reinterpret_cast<const u32x4 *>(Vh + (size_t)row * v_rs + 8 * c);
+        }
+        *reinterpret_cast<u32x4 *>(Qs + row * D + 8 * c) = q4;
+        *reinterpret_cast<u32x4 *>(Ks + row * D + 8 * (c ^ (row & (CPR - 1)))) = k4;
+        *reinterpret_cast<u32x4 *>(Vs + row * D + 8 * c) = v4;
+    }
+    __syncthreads();
     // scores (main.cu:189-197), masked entries -inf (main.cu:210-229); query i at position p sees keys p-L..p
     for (int idx = tid; idx < R * R; idx += nthr) {
         const int i = idx / R, j = idx % R, p = i + pos_off;
         float s = -INFINITY;
         if (i < rows && j <= p && p - j <= L) {
             float sum = 0.0f;
-            for (int t = 0; t < D; ++t)
-                sum += storage_product<BF16>(storage_to_f32<BF16>(Qh[(size_t)i * q_rs + t]), storage_to_f32<BF16>(Kh[(size_t)j * k_rs + t]));
+            for (int c = 0; c < CPR; ++c) {
+                const u32x4 qa = *reinterpret_cast<const u32x4 *>(Qs + i * D + 8 * c);
+                const u32x4 kb = *reinterpret_cast<const u32x4 *>(Ks + j * D + 8 * (c ^ (j & (CPR - 1))));
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const f32x2 pr = storage_product2<BF16>(qa[w], kb[w]);
+                    sum += pr[0];
+                    sum += pr[1];
+                }
+            }
             s = sum * scale;
             // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
             if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(p - j)));
@@ -252,19 +306,29 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
                 const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)(i + pos_off), (uint32_t)((j >> 2) & 1));
                 pj = dropout_keep_byte(d, 4 * (j >> 3) + (j & 3), drop_threshold) ? __fmul_rn(pj, drop_scale) : 0.0f;
             }
-            pj = storage_to_f32<BF16>(f32_to_storage<BF16>(pj));
         }
-        ex[idx] = pj;
+        const uint32_t bits = f32_to_storage<BF16>(pj);
+        pbits[idx] = bits | (bits << 16);       // (each thread overwrites only the element it has just read)
     }
     __syncthreads();
-    // weighted sum (main.cu:255-263), keys in ascending order; masked keys have p = 0 and add nothing
-    for (int idx = tid; idx < rows * D; idx += nthr) {
-        const int i = idx / D, t = idx % D, p = i + pos_off;
+    // weighted sum (main.cu:255-263), keys in ascending order; masked keys have p = 0 and add nothing.  A thread
+    // owns two neighbouring output elements of one row.
+    for (int idx = tid; idx < rows * (D / 2); idx += nthr) {
+        const int i = idx / (D / 2), t2 = idx % (D / 2), p = i + pos_off;
         const int lo = p - L > 0 ? p - L : 0;
-        float sum = 0.0f;
-        for (int j = lo; j <= p; ++j) sum += storage_product<BF16>(ex[i * R + j], storage_to_f32<BF16>(Vh[(size_t)j * v_rs + t]));
-        if (o32 != nullptr) o32[(size_t)i * D + t] = storage_to_f32<BF16>(f32_to_storage<BF16>(sum));
-        else Oh[(size_t)i * o_rs + t] = f32_to_storage<BF16>(sum);
+        float s0 = 0.0f, s1 = 0.0f;
+        for (int j = lo; j <= p; ++j) {
+            const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *reinterpret_cast<const uint32_t *>(Vs + j * D + 2 * t2));
+            s0 += pr[0];
+            s1 += pr[1];
+        }
+        const uint32_t packed = Num<BF16>::pack2(s0, s1);
+        if (o32 != nullptr) {
+            o32[(size_t)i * D + 2 * t2] = storage_to_f32<BF16>((uint16_t)(packed & 0xffffu));
+            o32[(size_t)i * D + 2 * t2 + 1] = storage_to_f32<BF16>((uint16_t)(packed >> 16));
+        } else {
+            *reinterpret_cast<uint32_t *>(Oh + (size_t)i * o_rs + 2 * t2) = packed;
+        }
     }
     __syncthreads();
 }
@@ -298,7 +362,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
     constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
     static_assert(INSTR % NW == 0, "tile must divide over the waves");
-    static_assert(NST >= 2 && NST <= 3 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
+    static_assert(NST >= 2 && NST <= 4 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
     typedef Num<BF16> N;
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -360,6 +424,18 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (taken == 0xffffffffu) break;
         item = (long long)taken;
     }
+#ifdef FA_TIMELINE
+    long long *tl = (g_fa_timeline != nullptr && tid == 0) ? g_fa_timeline + 16 * item : nullptr;
+    long long tl_generic = 0, tl_steady = 0;
+    if (tl != nullptr) {
+        unsigned hw;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+        unsigned xc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xc));
+        tl[0] = item; tl[1] = ((long long)(xc & 15u) << 32) | hw;
+    }
+#endif
+    FA_TL(2);
     int bh, qblock;
     // (GENERAL with key splits: consecutive list positions are the splits of one (head, query block))
     const int n_splits = GENERAL ? a.n_splits : 1;
@@ -751,9 +827,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     };
 
     if (any_tile) {             // (GENERAL: a split, or a block of rows that sees no key, may have no tile at all)
-    // ---- prologue: K(t0) .. K(t0+LA-1) resident before the first iteration
+    // ---- prologue: K(t0) .. K(t0+LA-1) and V(t0) .. V(t0+LA-3) requested before the first iteration (iteration
+    // i requests K(i+1+LA) and V(i-1+LA), and the first one is i = t0 - 1)
     issue_k(t0, 0);
     if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
+    if (LA > 2 && t0 + 2 <= t1) issue_k(t0 + 2, 2);
+    if (LA > 2) issue_v(t0, 0);
     wait_vm<0>();
     // Q has landed too (vmcnt is 0).  Touching the fragments here lets the compiler see that, so that it places
     // no vmcnt wait of its own inside the loop, where it would also wait for the asynchronous tile loads.
@@ -762,6 +841,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[b][s]));
     phase_barrier();
+    FA_TL(3);
 
     // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST
     // of its tensor, so the iteration reads K stage j % NST and V stage (j - 2) % NST; it issues the loads of
@@ -769,11 +849,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // Every wave executes every iteration (one barrier each); a wave whose own tile range does not cover all
     // three pieces runs the plain pieces it has, the others run the interleaved body.  The two kinds live in
     // separate loops: merging them under one branch makes the register allocator spill.
+    bool prev_full = false;     // the previous iteration requested both of its tiles
     auto finish_iteration = [&](bool full_issue) __attribute__((always_inline)) {
-        // what the next iteration reads must have landed; with three stages that was issued one iteration
-        // ago, so the loads issued just now may stay in flight
-        if (NST == 3 && full_issue) wait_vm<2 * IPW>();
+        // What the next iteration reads must have landed: that was requested LA - 1 iterations ago, so the
+        // requests of the LA - 1 most recent iterations may stay in flight (vmcnt counts requests, so this only
+        // holds while every one of those iterations made all of its 2 * IPW requests)
+        if (NST == 4 && full_issue && prev_full) wait_vm<4 * IPW>();
+        else if (NST >= 3 && full_issue) wait_vm<2 * IPW>();
         else wait_vm<0>();
+        prev_full = full_issue;
         phase_barrier();
     };
     auto generic_iteration = [&](int i, int j3) __attribute__((always_inline)) {
@@ -801,19 +885,30 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     for (; i <= t1 + 1; ++i) {            // fill: until NST consecutive iterations are steady and the stage is 0
         if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
         generic_iteration(i, j3);
+#ifdef FA_TIMELINE
+        ++tl_generic;
+#endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
     for (; i >= my_lo + 1 && i + NST - 1 <= my_hi - 1 && i <= t1 + 1; i += NST) {
         steady_iteration(IntC<0>{}, i);
         steady_iteration(IntC<1>{}, i + 1);
-        if (NST == 3) steady_iteration(IntC<2 % NST>{}, i + 2);
+        if (NST >= 3) steady_iteration(IntC<2 % NST>{}, i + 2);
+        if (NST >= 4) steady_iteration(IntC<3 % NST>{}, i + 3);
+#ifdef FA_TIMELINE
+        tl_steady += NST;
+#endif
     }
     for (j3 = 0; i <= t1 + 1; ++i) {      // drain
         generic_iteration(i, j3);
+#ifdef FA_TIMELINE
+        ++tl_generic;
+#endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
 
     }   // any_tile
+    FA_TL(4);
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
@@ -871,10 +966,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             if (a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
         }
     }
+    FA_TL(5);
     if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      f_rows, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
-                                     a.seed_lo, a.seed_hi, (uint32_t)bh, reinterpret_cast<float *>(smem));
+                                     a.seed_lo, a.seed_hi, (uint32_t)bh, smem);
+    FA_TL(6);
+#ifdef FA_TIMELINE
+    if (tl != nullptr) { tl[7] = tl_generic; tl[8] = tl_steady; tl[9] = ((long long)t0 << 32) | (unsigned)t1; }
+#endif
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
     if (a.queue != nullptr && tid == 0) {
@@ -948,13 +1048,16 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 // (The 8-wave general instantiations get two LDS stages instead of three: with three they come back from the
 // compiler with 270-350 bytes of spills whose reloads wait on the tile loads in flight -- c3's shape stored
 // [B,S,H,D] ran at 615 TFLOP/s, with two stages nothing spills and it runs at 940.)
+#ifndef FA_NST8
+#define FA_NST8 3
+#endif
 template <bool GENERAL, bool DROPOUT>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : 3)>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : FA_NST8)>(a, grid, stream); \
         return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
