@@ -22,7 +22,9 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 # HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
 # worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 424.1 MB read + 137.0 MB written.
-MEASURED_HBM_BYTES = {"c3": 561.1e6}
+MEASURED_HBM_BYTES = {"c3": 561.1e6, "c2": 68.2e6, "c4": 778.4e6}
+TRAFFIC_SOURCE = {"c3": "profiles/fa_fwd_pipelined_c3_pmc.md", "c2": "profiles/fa_fwd_pipelined_c2_pmc.md",
+                  "c4": "profiles/fa_fwd_pipelined_c4_pmc.md"}
 # the same for the two backward kernels together on c3's shape: 1756.4 MB read + 414.9 MB written
 MEASURED_BWD_HBM_BYTES = {"c3": 2171.3e6}
 
@@ -188,6 +190,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + sorted(DECODE_WORKLOADS))
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="before the warm-up steps, keep the GPU busy with the same kernel for this long: an idle MI355X "
+                         "raises its clock over some hundred milliseconds of load, and the timed steps are meant to "
+                         "measure the sustained rate (0 disables; reported as settle_ms)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline sample; 0 disables")
     ap.add_argument("--check-rows", type=int, default=1024, help="rows verified against the oracle; 0 disables")
     ap.add_argument("--sched", type=int, default=0, choices=(0, 1, 2, 3), help="0 library default, 1 dispatch, 2 persistent snake, 3 persistent queue")
@@ -243,6 +249,15 @@ def main():
         fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, out=out, lse=lse, sched=args.sched,
                                    alibi_slopes=tslopes, dropout_prob=args.dropout, seed=48)
 
+    # clock settle (untimed, reported): launches back to back until the wall clock says settle_ms have passed
+    settle_steps = 0
+    if args.settle_ms > 0:
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+            for _ in range(8):
+                step()
+            settle_steps += 8
+            torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -275,6 +290,7 @@ def main():
         "metric": ("attn fwd TFLOPS + % of fp16 MFMA peak, hd128 causal seq 8192, 1 GPU" if args.workload == "c3" and not variant
                    else f"attn fwd TFLOPS + % of MFMA peak, workload {args.workload}, 1 GPU"),
         "value": round(tflops, 2), "unit": "TFLOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_ms": args.settle_ms, "settle_steps": settle_steps,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D} "
@@ -287,6 +303,7 @@ def main():
         "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kernel_tflops / PEAK_TFLOPS, 4), "traffic": None if variant else MEASURED_HBM_BYTES.get(args.workload),
+                     "traffic_source": None if variant else TRAFFIC_SOURCE.get(args.workload),
                      "kernel_ms_avg": round(avg_kernel_ms, 5), "kernel_ms_median": round(float(np.median(kernel_ms)), 5),
                      "kernel_ms_min": round(float(np.min(kernel_ms)), 5)},
     }

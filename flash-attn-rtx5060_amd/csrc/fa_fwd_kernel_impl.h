@@ -126,7 +126,11 @@ __device__ __forceinline__ void dma_16(const char *base, uint32_t voff, uint32_t
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
 }
+#ifdef FA_EXP_NOBAR          /* timing experiment only: no workgroup barrier, races */
+__device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+#else
 __device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+#endif
 
 template <int V> struct IntC { static constexpr int value = V; };
 
@@ -137,7 +141,7 @@ template <int V> struct IntC { static constexpr int value = V; };
 // shader clock counter at the same five points.
 #ifdef FA_TIMELINE
 __device__ long long *g_fa_timeline = nullptr;
-#define FA_TL(slot) do { if (tl != nullptr) { tl[slot] = (long long)__builtin_amdgcn_s_memrealtime(); tl[slot + 8] = (long long)__builtin_amdgcn_s_memtime(); } } while (0)
+#define FA_TL(slot) do { if (tid == 0) { tl_lds[slot] = (long long)__builtin_amdgcn_s_memrealtime(); tl_lds[slot + 8] = (long long)__builtin_amdgcn_s_memtime(); } } while (0)
 #else
 #define FA_TL(slot) do { } while (0)
 #endif
@@ -384,7 +388,16 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcd));
         xcd &= 7u;
     }
-    volatile unsigned *next_slot = reinterpret_cast<volatile unsigned *>(smem + 2 * NST * TILEB);
+    // next_slot[0] broadcasts the list position a queue-scheduled workgroup has taken; next_slot[1] holds the
+    // value of the own XCD's counter that was fetched ahead of time (during the previous item's epilogue), or
+    // kNoPrefetch
+    volatile __attribute__((address_space(3))) unsigned *next_slot =
+        (volatile __attribute__((address_space(3))) unsigned *)(uintptr_t)(lds0 + 2 * NST * TILEB);
+    constexpr unsigned kNoPrefetch = 0xffffffffu;
+    if (a.queue != nullptr) {
+        if (tid == 0) next_slot[1] = kNoPrefetch;
+        __syncthreads();
+    }
     for (int pass = 0;; ++pass) {
     long long item;
     if (a.queue == nullptr) {
@@ -399,7 +412,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             // updated: a workgroup that finds nothing left then pays for one read instead of eight updates in
             // a row, on counters that every other leaving workgroup updates at the same time.)
             unsigned found = 0xffffffffu;
-            const long long own = (long long)atomicAdd(&a.queue[xcd], 1u) * 8 + xcd;
+            unsigned ticket = next_slot[1];
+            if (ticket == kNoPrefetch) ticket = atomicAdd(&a.queue[xcd], 1u);
+            next_slot[1] = kNoPrefetch;
+            const long long own = (long long)ticket * 8 + xcd;
             if (own < a.n_items) found = (unsigned)own;
             while (found == 0xffffffffu) {
                 unsigned cnt[8];
@@ -425,14 +441,16 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         item = (long long)taken;
     }
 #ifdef FA_TIMELINE
-    long long *tl = (g_fa_timeline != nullptr && tid == 0) ? g_fa_timeline + 16 * item : nullptr;
-    long long tl_generic = 0, tl_steady = 0;
-    if (tl != nullptr) {
-        unsigned hw;
+    // (the words are collected in LDS behind the queue slot and copied out at the end of the item, so that no
+    // pointer stays live in registers across the tile loop)
+    volatile __attribute__((address_space(3))) long long *tl_lds =
+        (volatile __attribute__((address_space(3))) long long *)(uintptr_t)(lds0 + 2 * NST * TILEB + 64);
+    const long long tl_item = item;
+    if (tid == 0) {
+        unsigned hw, xc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-        unsigned xc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xc));
-        tl[0] = item; tl[1] = ((long long)(xc & 15u) << 32) | hw;
+        tl_lds[0] = item; tl_lds[1] = ((long long)(xc & 15u) << 32) | hw; tl_lds[7] = 0; tl_lds[8] = 0;
     }
 #endif
     FA_TL(2);
@@ -771,8 +789,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         float alpha[RB], nmc[RB];
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
+#ifdef FA_EXP_NOMAX      /* timing experiment only: no row maximum, wrong results */
+            alpha[b] = 1.0f; moved[b] = false; nmc[b] = -6.0f;
+#else
             alpha[b] = new_reference(b, row_max(b), moved[b]);
             nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * cs;
+#endif
         }
         uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
         f32x16 nx[RB][2];                          // S^T(tile+1)
@@ -886,7 +908,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
         generic_iteration(i, j3);
 #ifdef FA_TIMELINE
-        ++tl_generic;
+        if (tid == 0) tl_lds[7] = tl_lds[7] + 1;
 #endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
@@ -896,19 +918,25 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (NST >= 3) steady_iteration(IntC<2 % NST>{}, i + 2);
         if (NST >= 4) steady_iteration(IntC<3 % NST>{}, i + 3);
 #ifdef FA_TIMELINE
-        tl_steady += NST;
+        if (tid == 0) tl_lds[8] = tl_lds[8] + NST;
 #endif
     }
     for (j3 = 0; i <= t1 + 1; ++i) {      // drain
         generic_iteration(i, j3);
 #ifdef FA_TIMELINE
-        ++tl_generic;
+        if (tid == 0) tl_lds[7] = tl_lds[7] + 1;
 #endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
 
     }   // any_tile
     FA_TL(4);
+    // Queue schedule: the counter round trip for the NEXT item (2.3 us) runs in the shadow of this item's
+    // epilogue; its result is parked in LDS for the take at the top of the loop.  (A workgroup thus takes one
+    // list position more than it processes when the list runs out; the counters only have to be monotonic, and
+    // the last workgroup to leave rewinds them.)
+    unsigned ticket_ahead = 0;
+    if (a.queue != nullptr && tid == 0) ticket_ahead = atomicAdd(&a.queue[xcd], 1u);
 
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
@@ -971,9 +999,14 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      f_rows, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
                                      a.seed_lo, a.seed_hi, (uint32_t)bh, smem);
+    if (a.queue != nullptr && tid == 0) next_slot[1] = ticket_ahead;
     FA_TL(6);
 #ifdef FA_TIMELINE
-    if (tl != nullptr) { tl[7] = tl_generic; tl[8] = tl_steady; tl[9] = ((long long)t0 << 32) | (unsigned)t1; }
+    if (tid == 0 && g_fa_timeline != nullptr) {
+        tl_lds[9] = ((long long)t0 << 32) | (unsigned)t1;
+        for (int w = 0; w < 16; ++w) g_fa_timeline[16 * tl_item + w] = tl_lds[w];
+    }
+    __syncthreads();
 #endif
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
@@ -1026,7 +1059,11 @@ template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT,
 hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
-    const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the word that broadcasts a queue position
+#ifdef FA_TIMELINE
+    const size_t smem = 2 * NST * TILEB + 64 + 128;
+#else
+    const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the two words of the queue schedule
+#endif
     auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST>;
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
