@@ -88,6 +88,36 @@ template <> struct Num<true> {
     }
 };
 
+// The same matrix instructions with their register files pinned, for the 64-rows-per-wave shape (one wave per
+// SIMD, 512 registers): the O^T accumulators and the Q^T fragments live in the accumulation registers, which
+// only matrix instructions touch, the S^T accumulators and everything the vector ALU works on in the ordinary
+// ones.  Left to the register allocator, values wander between the two files (about 240 moves per tile).
+// Written as inline assembly the compiler no longer sees a matrix instruction and inserts no wait states for
+// it: every place where a result is read by a vector instruction within about twenty cycles carries an
+// explicit s_nop (mfma_result_wait), and results are reused as accumulators only several matrix
+// instructions later.
+template <bool BF16> struct PinnedMfma {
+    // S^T block: D in ordinary registers, B operand (Q^T) in accumulation registers; first of a chain: C = 0
+    static __device__ __forceinline__ void qk_first(f32x16 &d, u32x4 a, u32x4 b)
+    {
+        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+    }
+    static __device__ __forceinline__ void qk_next(f32x16 &d, u32x4 a, u32x4 b)
+    {
+        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+    }
+    // O^T block: accumulator in accumulation registers, operands in ordinary registers
+    static __device__ __forceinline__ void pv(f32x16 &acc, u32x4 a, u32x4 b)
+    {
+        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    }
+};
+// wait states between a pinned matrix instruction and a vector instruction that reads its result
+__device__ __forceinline__ void mfma_result_wait() { asm volatile("s_nop 15\n\ts_nop 9" ::: "memory"); }
+
 // 16-byte-chunk swizzles.  A tile row holds CPR = D/8 chunks.
 // K is read with ds_read_b128 by 16 lanes holding 16 consecutive rows and one
 // logical chunk: those must land on 16 different 16-byte bank groups.
@@ -536,6 +566,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                                        Qh + (GENERAL ? (size_t)row_head[b] * a.q_hs : 0) + (size_t)row_pos[b] * q_rs + 16 * s + 8 * half)
                                  : u32x4{0, 0, 0, 0};
 
+#ifdef FA_TIMELINE      /* word 15: the wall clock when this wave's Q fragments have landed */
+    wait_vm<0>();
+    if (tid == 0) tl_lds[15] = (long long)__builtin_amdgcn_s_memrealtime();
+#endif
     const int rows_in_block = pack > 1 ? S : S - q0 < BR ? S - q0 : BR;
     int t0, t1;                 // key tiles visited by the workgroup
     fa_tile_range(Sk, kBlockKeys, a.L, a.R, block_pos0 + pos_off, rows_in_block, &t0, &t1);
@@ -687,9 +721,24 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     };
     auto scale_o = [&](int b, float alpha) __attribute__((always_inline)) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db) {
+            if (RB == 2) {
+                // O^T lives in accumulation registers, the vector ALU cannot read those: copy out, scale, copy
+                // back.  The empty statements tie every copy to this (rare) branch; without them the compiler
+                // moves the copies in front of the branch, into every iteration.
+                asm volatile("" : "+a"(o[b][db]));
+                f32x16 t = o[b][db];
+                asm volatile("" : "+v"(t));
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[b][db][r] *= alpha;
+                for (int r = 0; r < 16; ++r) t[r] *= alpha;
+                asm volatile("" : "+v"(t));
+                o[b][db] = t;
+                asm volatile("" : "+a"(o[b][db]));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[b][db][r] *= alpha;
+            }
+        }
     };
     auto p_operand = [&](int b, int t2) __attribute__((always_inline)) {
         return u32x4{pk[b][4 * t2], pk[b][4 * t2 + 1], pk[b][4 * t2 + 2], pk[b][4 * t2 + 3]};
@@ -709,9 +758,13 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             if (n + 2 < NPV) fr[n + 2] = read_v(vs, n + 2);
             const int t2 = n / DB, db = n % DB;
 #pragma unroll
-            for (int b = 0; b < RB; ++b) o[b][db] = N::mfma(fr[n], p_operand(b, t2), o[b][db]);
+            for (int b = 0; b < RB; ++b) {
+                if (RB == 2) PinnedMfma<BF16>::pv(o[b][db], fr[n], p_operand(b, t2));
+                else o[b][db] = N::mfma(fr[n], p_operand(b, t2), o[b][db]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (RB == 2) mfma_result_wait();       // the epilogue may follow
     };
     auto qk_plain = [&](int kstage) __attribute__((always_inline)) {
         const uint32_t ks = kstage * TILEB;
@@ -727,9 +780,13 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int n = 0; n < NQK; ++n) {
             if (n + 2 < NQK) fr[n + 2] = read_k(ks, n + 2);
 #pragma unroll
-            for (int b = 0; b < RB; ++b) sx[b][n & 1] = N::mfma(fr[n], qf[b][n >> 1], sx[b][n & 1]);
+            for (int b = 0; b < RB; ++b) {
+                if (RB == 2) PinnedMfma<BF16>::qk_next(sx[b][n & 1], fr[n], qf[b][n >> 1]);
+                else sx[b][n & 1] = N::mfma(fr[n], qf[b][n >> 1], sx[b][n & 1]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (RB == 2) mfma_result_wait();
     };
     // dropout decisions of the tile whose exponentials come next: per row block and key block the sixteen
     // bytes for this lane's sixteen keys
@@ -806,11 +863,14 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             for (int b = 0; b < RB; ++b) {
                 if (g < NPV) {
                     const int t2 = g / DB, db = g % DB;
-                    o[b][db] = N::mfma(fr[g], p_operand(b, t2), o[b][db]);
+                    if (RB == 2) PinnedMfma<BF16>::pv(o[b][db], fr[g], p_operand(b, t2));
+                    else o[b][db] = N::mfma(fr[g], p_operand(b, t2), o[b][db]);
                 } else {
                     const int n = g - NPV;
                     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n < 2 ? zero : nx[b][n & 1]);
+                    if (RB == 2 && n < 2) PinnedMfma<BF16>::qk_first(nx[b][n & 1], fr[g], qf[b][n >> 1]);
+                    else if (RB == 2) PinnedMfma<BF16>::qk_next(nx[b][n & 1], fr[g], qf[b][n >> 1]);
+                    else nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n < 2 ? zero : nx[b][n & 1]);
                 }
                 // softmax work riding along: the 16*RB element pairs of this tile spread over the NF*RB matrix
                 // instructions, row block 0 first (its registers are free again when S^T(tile+1) is born)
@@ -838,6 +898,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (RB == 2) mfma_result_wait();           // S^T(tile+1) is read by vector instructions next
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             if (moved[b]) scale_o(b, alpha[b]);    // rare; PV(tile-1) has been issued in full by now
@@ -861,7 +922,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
     for (int b = 0; b < RB; ++b)
 #pragma unroll
-        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[b][s]));
+        for (int s = 0; s < KS; ++s) {
+            // (64 rows per wave: from here on the fragments live in accumulation registers, where the pinned
+            // matrix instructions read them; in ordinary registers each use would cost four copies)
+            if (RB == 2) asm volatile("" : "+a"(qf[b][s]));
+            else asm volatile("" : "+v"(qf[b][s]));
+        }
     phase_barrier();
     FA_TL(3);
 
@@ -1088,12 +1154,16 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 #ifndef FA_NST8
 #define FA_NST8 3
 #endif
+#ifndef FA_ROWS64       /* 1: the 64-rows-per-wave shape for head dimension 128, contiguous layout (under evaluation) */
+#define FA_ROWS64 0
+#endif
 template <bool GENERAL, bool DROPOUT>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
+        if (shape == 0 && FA_ROWS64 && !GENERAL && DD == 128 && !AL) return launch<BF != 0, DD, MK != 0, false, false, false, 4, (FA_ROWS64 ? 2 : 1), 3>(a, grid, stream); \
         if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : FA_NST8)>(a, grid, stream); \
         return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
