@@ -156,11 +156,7 @@ __device__ __forceinline__ void dma_16(const char *base, uint32_t voff, uint32_t
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
 }
-#ifdef FA_EXP_NOBAR          /* timing experiment only: no workgroup barrier, races */
-__device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-#else
 __device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-#endif
 
 template <int V> struct IntC { static constexpr int value = V; };
 
@@ -846,12 +842,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         float alpha[RB], nmc[RB];
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
-#ifdef FA_EXP_NOMAX      /* timing experiment only: no row maximum, wrong results */
-            alpha[b] = 1.0f; moved[b] = false; nmc[b] = -6.0f;
-#else
             alpha[b] = new_reference(b, row_max(b), moved[b]);
             nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * cs;
-#endif
         }
         uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
         f32x16 nx[RB][2];                          // S^T(tile+1)
