@@ -414,23 +414,19 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcd));
         xcd &= 7u;
     }
-    // next_slot[0] broadcasts the list position a queue-scheduled workgroup has taken; next_slot[1] holds the
-    // value of the own XCD's counter that was fetched ahead of time (during the previous item's epilogue), or
-    // kNoPrefetch
+    // next_slot broadcasts the list position a queue-scheduled workgroup has taken
     volatile __attribute__((address_space(3))) unsigned *next_slot =
         (volatile __attribute__((address_space(3))) unsigned *)(uintptr_t)(lds0 + 2 * NST * TILEB);
-    constexpr unsigned kNoPrefetch = 0xffffffffu;
-    if (a.queue != nullptr) {
-        if (tid == 0) next_slot[1] = kNoPrefetch;
-        __syncthreads();
-    }
-    for (int pass = 0;; ++pass) {
-    long long item;
-    if (a.queue == nullptr) {
-        if ((long long)pass * G >= a.n_items) break;
-        item = (long long)pass * G + ((pass & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x);
-        if (item >= a.n_items) continue;
-    } else {
+    constexpr unsigned kNoTicket = 0xffffffffu;
+    // The work item of pass `pass_no` of this workgroup, or -1 when its work is done (list positions fit 31
+    // bits, the host checks that).  Queue schedule: `ticket` is the value of the own XCD's counter when thread 0
+    // has fetched it ahead of time, or kNoTicket.
+    auto take_item = [&](int pass_no, unsigned ticket) __attribute__((always_inline)) -> int {
+        if (a.queue == nullptr) {
+            const long long base = (long long)pass_no * G;
+            const long long it = base + ((pass_no & 1) ? G - 1 - (int)blockIdx.x : (int)blockIdx.x);
+            return it < a.n_items ? (int)it : -1;     // (an odd pass may leave this workgroup out; the next is empty then)
+        }
         if (tid == 0) {
             // own XCD's list first; when that is exhausted, help the others (this also makes the result
             // independent of how the hardware spreads the workgroups over the XCDs)
@@ -438,9 +434,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             // updated: a workgroup that finds nothing left then pays for one read instead of eight updates in
             // a row, on counters that every other leaving workgroup updates at the same time.)
             unsigned found = 0xffffffffu;
-            unsigned ticket = next_slot[1];
-            if (ticket == kNoPrefetch) ticket = atomicAdd(&a.queue[xcd], 1u);
-            next_slot[1] = kNoPrefetch;
+            if (ticket == kNoTicket) ticket = atomicAdd(&a.queue[xcd], 1u);
             const long long own = (long long)ticket * 8 + xcd;
             if (own < a.n_items) found = (unsigned)own;
             while (found == 0xffffffffu) {
@@ -461,11 +455,17 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
         __syncthreads();
         // uniform by construction: say so, or everything derived from the item lives in vector registers
-        const unsigned taken = (unsigned)__builtin_amdgcn_readfirstlane((int)*next_slot);
+        const int taken = __builtin_amdgcn_readfirstlane((int)*next_slot);
         __syncthreads();
-        if (taken == 0xffffffffu) break;
-        item = (long long)taken;
-    }
+        return taken;
+    };
+    // The next work item is taken before the epilogue of the current one, and (contiguous layout) its Q^T
+    // fragments and first K tiles are requested there: the 3-5 us their first bytes take to arrive from HBM lie
+    // behind the epilogue instead of in front of the next tile loop.
+    u32x4 qf[RB][KS];
+    bool next_requested = false;
+    int item = take_item(0, kNoTicket);
+    for (int pass = 0; item >= 0; ++pass) {
 #ifdef FA_TIMELINE
     // (the words are collected in LDS behind the queue slot and copied out at the end of the item, so that no
     // pointer stays live in registers across the tile loop)
@@ -483,11 +483,13 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     int bh, qblock;
     // (GENERAL with key splits: consecutive list positions are the splits of one (head, query block))
     const int n_splits = GENERAL ? a.n_splits : 1;
-    const int split = n_splits > 1 ? (int)(item % n_splits) : 0;
+    // (list positions fit 31 bits, the host checks that: 32-bit divisions)
+    const unsigned head_item = n_splits > 1 ? (unsigned)item / (unsigned)n_splits : (unsigned)item;
+    const int split = n_splits > 1 ? (int)((unsigned)item - head_item * (unsigned)n_splits) : 0;
     // (GENERAL, packed groups: an item is a (batch, K/V head); its rows are the queries of all query heads
     // of that K/V head, head after head -- few queries against long keys read K and V once per group)
     const int pack = GENERAL ? a.pack : 1;
-    fa_item_decode(n_splits > 1 ? item / n_splits : item, pack > 1 ? a.BH / pack : a.BH, a.n_qblocks, a.descending, &bh, &qblock);
+    fa_item_decode((long long)head_item, pack > 1 ? a.BH / pack : a.BH, a.n_qblocks, a.descending, &bh, &qblock);
     const int S = a.S;
     // GENERAL: Sk keys; query i sits at key position i + pos_off (the queries are the last S positions), which
     // is what masks, the ALiBi distance and the dropout decision see.
@@ -553,14 +555,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     }
 
     // Q^T fragments: B operand, lane = (query l32, head-dim slice 8*half..+7 of each 16)
-    u32x4 qf[RB][KS];
+    if (!next_requested) {
 #pragma unroll
-    for (int b = 0; b < RB; ++b)
+        for (int b = 0; b < RB; ++b)
 #pragma unroll
-        for (int s = 0; s < KS; ++s)
-            qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(
-                                       Qh + (GENERAL ? (size_t)row_head[b] * a.q_hs : 0) + (size_t)row_pos[b] * q_rs + 16 * s + 8 * half)
-                                 : u32x4{0, 0, 0, 0};
+            for (int s = 0; s < KS; ++s)
+                qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(
+                                           Qh + (GENERAL ? (size_t)row_head[b] * a.q_hs : 0) + (size_t)row_pos[b] * q_rs + 16 * s + 8 * half)
+                                     : u32x4{0, 0, 0, 0};
+    }
 
 #ifdef FA_TIMELINE      /* word 15: the wall clock when this wave's Q fragments have landed */
     wait_vm<0>();
@@ -611,20 +614,22 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         const int last = Sk - 1 - tile * kBlockKeys, src_row = row < last ? row : last;
         return (uint32_t)(src_row * (rs * 2) + ((pos ^ (is_k ? k_swz<CPR>(row) : v_swz<CPR>(row))) << 4));
     };
-    auto issue_k = [&](int tile, int stage) __attribute__((always_inline)) {
-        const char *src = reinterpret_cast<const char *>(Kh) + (size_t)tile * (kBlockKeys * 2) * k_rs;
+    auto issue_k_from = [&](const uint16_t *k_head, int tile, int stage) __attribute__((always_inline)) {
+        const char *src = reinterpret_cast<const char *>(k_head) + (size_t)tile * (kBlockKeys * 2) * k_rs;
         const bool ragged = GENERAL && (tile + 1) * kBlockKeys > Sk;
 #pragma unroll
         for (int i = 0; i < IPW; ++i)
             dma_16(src, ragged ? ragged_source(tile, i, k_rs, true) : gk[i], lds0 + stage * TILEB + (i * NW + wave) * 1024);
     };
-    auto issue_v = [&](int tile, int stage) __attribute__((always_inline)) {
-        const char *src = reinterpret_cast<const char *>(Vh) + (size_t)tile * (kBlockKeys * 2) * v_rs;
+    auto issue_k = [&](int tile, int stage) __attribute__((always_inline)) { issue_k_from(Kh, tile, stage); };
+    auto issue_v_from = [&](const uint16_t *v_head, int tile, int stage) __attribute__((always_inline)) {
+        const char *src = reinterpret_cast<const char *>(v_head) + (size_t)tile * (kBlockKeys * 2) * v_rs;
         const bool ragged = GENERAL && (tile + 1) * kBlockKeys > Sk;
 #pragma unroll
         for (int i = 0; i < IPW; ++i)
             dma_16(src, ragged ? ragged_source(tile, i, v_rs, false) : gv[i], lds0 + LDS_V + stage * TILEB + (i * NW + wave) * 1024);
     };
+    auto issue_v = [&](int tile, int stage) __attribute__((always_inline)) { issue_v_from(Vh, tile, stage); };
     // skip / edge / free classification of a key tile for this wave (GENERAL: a tile that reaches past the
     // end of the sequence is an edge tile)
     auto tile_class = [&](int tile) __attribute__((always_inline)) {
@@ -901,13 +906,17 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
     };
 
+    unsigned ticket_ahead = kNoTicket;      // thread 0 only
     if (any_tile) {             // (GENERAL: a split, or a block of rows that sees no key, may have no tile at all)
     // ---- prologue: K(t0) .. K(t0+LA-1) and V(t0) .. V(t0+LA-3) requested before the first iteration (iteration
     // i requests K(i+1+LA) and V(i-1+LA), and the first one is i = t0 - 1)
-    issue_k(t0, 0);
-    if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
-    if (LA > 2 && t0 + 2 <= t1) issue_k(t0 + 2, 2);
-    if (LA > 2) issue_v(t0, 0);
+    if (!next_requested) {
+        issue_k(t0, 0);
+        if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
+        if (LA > 2 && t0 + 2 <= t1) issue_k(t0 + 2, 2);
+        if (LA > 2) issue_v(t0, 0);
+    }
+    next_requested = false;
     wait_vm<0>();
     // Q has landed too (vmcnt is 0).  Touching the fragments here lets the compiler see that, so that it places
     // no vmcnt wait of its own inside the loop, where it would also wait for the asynchronous tile loads.
@@ -930,13 +939,16 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // three pieces runs the plain pieces it has, the others run the interleaved body.  The two kinds live in
     // separate loops: merging them under one branch makes the register allocator spill.
     bool prev_full = false;     // the previous iteration requested both of its tiles
-    auto finish_iteration = [&](bool full_issue) __attribute__((always_inline)) {
+    auto finish_iteration = [&](bool full_issue, bool past_last_request) __attribute__((always_inline)) {
         // What the next iteration reads must have landed: that was requested LA - 1 iterations ago, so the
         // requests of the LA - 1 most recent iterations may stay in flight (vmcnt counts requests, so this only
         // holds while every one of those iterations made all of its 2 * IPW requests)
         if (NST == 4 && full_issue && prev_full) wait_vm<4 * IPW>();
         else if (NST >= 3 && full_issue) wait_vm<2 * IPW>();
-        else wait_vm<0>();
+        // (the last iterations of an item, those past the request for V(t1), request nothing, and the one before
+        // them has waited for everything: they do not wait, so that the counter fetched there for the next
+        // item stays in flight)
+        else if (!past_last_request) wait_vm<0>();
         prev_full = full_issue;
         phase_barrier();
     };
@@ -949,7 +961,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(jm2);
         if (my_lo <= i && i <= my_hi) softmax_plain(i);
         if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3);
-        finish_iteration(more_k && more_v);
+        finish_iteration(more_k && more_v, tv > t1);
     };
     auto steady_iteration = [&](auto J3, int i) __attribute__((always_inline)) {
         constexpr int j3 = decltype(J3)::value;
@@ -959,10 +971,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (more_k) issue_k(tk, jm1);
         if (more_v) issue_v(tv, jm3);
         steady(IntC<j3>{}, IntC<jm2>{}, i);
-        finish_iteration(more_k && more_v);
+        finish_iteration(more_k && more_v, false);
     };
     int i = t0 - 1, j3 = 0;
-    for (; i <= t1 + 1; ++i) {            // fill: until NST consecutive iterations are steady and the stage is 0
+    for (; i < t1; ++i) {                 // fill: until NST consecutive iterations are steady and the stage is 0
         if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
         generic_iteration(i, j3);
 #ifdef FA_TIMELINE
@@ -979,7 +991,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (tid == 0) tl_lds[8] = tl_lds[8] + NST;
 #endif
     }
-    for (j3 = 0; i <= t1 + 1; ++i) {      // drain
+    for (; i < t1; ++i) {                 // drain, up to the last two iterations
+        generic_iteration(i, j3);
+        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+    }
+    // Queue schedule: the counter round trip for the NEXT item (2.3 us) runs behind the last two iterations.
+    // (Between two loops on purpose: as a branch inside generic_iteration the same statement costs the whole
+    // kernel fifty registers.)
+    if (a.queue != nullptr && tid == 0) ticket_ahead = atomicAdd(&a.queue[xcd], 1u);
+    for (; i <= t1 + 1; ++i) {            // the last two iterations (three stages: they request nothing any more)
         generic_iteration(i, j3);
 #ifdef FA_TIMELINE
         if (tid == 0) tl_lds[7] = tl_lds[7] + 1;
@@ -989,13 +1009,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     }   // any_tile
     FA_TL(4);
-    // Queue schedule: the counter round trip for the NEXT item (2.3 us) runs in the shadow of this item's
-    // epilogue; its result is parked in LDS for the take at the top of the loop.  (A workgroup thus takes one
-    // list position more than it processes when the list runs out; the counters only have to be monotonic, and
-    // the last workgroup to leave rewinds them.)
-    unsigned ticket_ahead = 0;
-    if (a.queue != nullptr && tid == 0) ticket_ahead = atomicAdd(&a.queue[xcd], 1u);
-
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
     // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32
@@ -1003,6 +1016,28 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // fa_fwd_params.exact_first_rows switches the path off)
     const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off >= 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
     const int f_rows = !faithful ? 0 : !GENERAL ? kFaithfulRows : (kFaithfulRows - pos_off < S ? kFaithfulRows - pos_off : S);
+    // ---- the next work item, and the first requests for it
+    const int next_item = take_item(pass + 1, ticket_ahead);
+    // (an item that ends with the first-rows path uses the K stages' LDS for it: nothing is requested then)
+    if (!GENERAL && RB == 1 && next_item >= 0 && !faithful) {
+        int nbh, nqb, nt0, nt1;
+        fa_item_decode(next_item, a.BH, a.n_qblocks, a.descending, &nbh, &nqb);
+        const size_t noff = (size_t)nbh * S * D;
+        const int nq0 = nqb * BR;
+        fa_tile_range(S, kBlockKeys, a.L, a.R, nq0, S - nq0 < BR ? S - nq0 : BR, &nt0, &nt1);
+        // (every LDS stage is free: the last iteration ended with a barrier)
+        issue_k_from(a.K + noff, nt0, 0);
+        if (LA > 1 && nt0 + 1 <= nt1) issue_k_from(a.K + noff, nt0 + 1, 1);
+        if (LA > 2 && nt0 + 2 <= nt1) issue_k_from(a.K + noff, nt0 + 2, 2);
+        if (LA > 2) issue_v_from(a.V + noff, nt0, 0);
+        // (S is a multiple of 128: a wave has all its rows or none; one without rows never uses its fragments and
+        // reads those of the block's first wave, so that no select has to wait for the data)
+        const int nrow = nq0 + (nq0 + wave * WR < S ? wave * WR : 0) + l32;
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            qf[0][s] = *reinterpret_cast<const u32x4 *>(a.Q + noff + (size_t)nrow * D + 16 * s + 8 * half);
+        next_requested = true;
+    }
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
     // own keys), which fa_combine_splits merges.
     float *o_part = nullptr, *lse_part = nullptr;
@@ -1057,7 +1092,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      f_rows, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
                                      a.seed_lo, a.seed_hi, (uint32_t)bh, smem);
-    if (a.queue != nullptr && tid == 0) next_slot[1] = ticket_ahead;
     FA_TL(6);
 #ifdef FA_TIMELINE
     if (tid == 0 && g_fa_timeline != nullptr) {
@@ -1066,6 +1100,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     }
     __syncthreads();
 #endif
+    item = next_item;
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
     if (a.queue != nullptr && tid == 0) {
@@ -1149,13 +1184,19 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 #ifndef FA_ROWS64       /* 1: the 64-rows-per-wave shape for head dimension 128, contiguous layout (under evaluation) */
 #define FA_ROWS64 0
 #endif
+#if FA_ROWS64
+#define FA_ROWS64_CASE(BF, DD, MK, AL) \
+    if (shape == 0 && !GENERAL && DD == 128 && !AL) return launch<BF != 0, DD, MK != 0, false, false, false, 4, 2, 3>(a, grid, stream);
+#else
+#define FA_ROWS64_CASE(BF, DD, MK, AL)
+#endif
 template <bool GENERAL, bool DROPOUT>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
-        if (shape == 0 && FA_ROWS64 && !GENERAL && DD == 128 && !AL) return launch<BF != 0, DD, MK != 0, false, false, false, 4, (FA_ROWS64 ? 2 : 1), 3>(a, grid, stream); \
+        FA_ROWS64_CASE(BF, DD, MK, AL) \
         if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : FA_NST8)>(a, grid, stream); \
         return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
@@ -1163,6 +1204,7 @@ hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, in
     FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)
 #undef FA_CASES
 #undef FA_CASE
+#undef FA_ROWS64_CASE
     return hipErrorInvalidValue;
 }
 

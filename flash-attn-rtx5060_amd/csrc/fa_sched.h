@@ -64,19 +64,22 @@ FA_HD int fa_tile_class(int block_keys, int L, int R, int q_begin, int rows, int
 #define FA_HEAD_GROUP 8
 FA_HD void fa_item_decode(long long item, int BH, int n_qblocks, int descending, int *bh, int *qblock)
 {
-    const long long per_group = (long long)FA_HEAD_GROUP * n_qblocks;
-    const int full_groups = BH / FA_HEAD_GROUP;
-    int group = (int)(item / per_group);
-    int heads_here = FA_HEAD_GROUP;
-    long long rem = item - (long long)group * per_group;
+    // (list positions and FA_HEAD_GROUP * n_qblocks fit 31 bits, which the host checks before a launch: 32-bit
+    // unsigned divisions, a few instructions each on the GPU where a 64-bit one is a long subroutine that every
+    // work item would pay for three times)
+    const unsigned it = (unsigned)item;
+    const unsigned per_group = (unsigned)FA_HEAD_GROUP * (unsigned)n_qblocks;
+    const unsigned full_groups = (unsigned)BH / FA_HEAD_GROUP;
+    unsigned group = it / per_group;
+    unsigned heads_here = FA_HEAD_GROUP;
     if (group >= full_groups) {          // the last, smaller group
         group = full_groups;
-        heads_here = BH - full_groups * FA_HEAD_GROUP;
-        rem = item - (long long)full_groups * per_group;
+        heads_here = (unsigned)BH - full_groups * FA_HEAD_GROUP;
     }
-    const int rank = (int)(rem / heads_here);
-    *bh = group * FA_HEAD_GROUP + (int)(rem % heads_here);
-    *qblock = descending ? (n_qblocks - 1 - rank) : rank;
+    const unsigned rem = it - group * per_group;
+    const unsigned rank = rem / heads_here;
+    *bh = (int)(group * FA_HEAD_GROUP + (rem - rank * heads_here));
+    *qblock = descending ? (n_qblocks - 1 - (int)rank) : (int)rank;
 }
 
 #endif
