@@ -1175,11 +1175,14 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 // shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
 // (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
 // answers it with about 500 AGPR<->VGPR moves per tile.)
-// (The 8-wave general instantiations get two LDS stages instead of three: with three they come back from the
-// compiler with 270-350 bytes of spills whose reloads wait on the tile loads in flight -- c3's shape stored
-// [B,S,H,D] ran at 615 TFLOP/s, with two stages nothing spills and it runs at 940.)
+// (The 8-wave general instantiations get two LDS stages instead of three: a third buys nothing measurable --
+// c3's shape stored [B,S,H,D] runs at 925 TFLOP/s with two and 929 with three, c2's at 553 against 514 -- and
+// two leave LDS for a second workgroup of the small shapes.)
 #ifndef FA_NST8
 #define FA_NST8 3
+#endif
+#ifndef FA_NST8_GENERAL
+#define FA_NST8_GENERAL 2
 #endif
 #ifndef FA_ROWS64       /* 1: the 64-rows-per-wave shape for head dimension 128, contiguous layout (under evaluation) */
 #define FA_ROWS64 0
@@ -1197,7 +1200,7 @@ hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, in
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
         FA_ROWS64_CASE(BF, DD, MK, AL) \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? 2 : FA_NST8)>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? FA_NST8_GENERAL : FA_NST8)>(a, grid, stream); \
         return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
