@@ -119,7 +119,10 @@ def test_schedules_agree_bitwise(fa):
     """All schedules run the same per-item code: their outputs must be identical bit for bit, launch after
     launch (the work queue rewinds itself at the end of every launch that uses it)."""
     import torch
-    for shape, dtype, causal, wl in (((2, 8, 1024, 128), 0, True, -1), ((2, 40, 4096, 64), 1, True, 300), ((3, 5, 640, 64), 0, False, -1)):
+    for shape, dtype, causal, wl in (((2, 8, 1024, 128), 0, True, -1), ((2, 40, 4096, 64), 1, True, 300), ((3, 5, 640, 64), 0, False, -1),
+                                      # several passes over the resident grid, the last block of every head half empty:
+                                      # what a workgroup requests ahead for its next item must be that item's data
+                                      ((8, 40, 384, 128), 0, True, -1), ((4, 16, 2176, 128), 1, False, -1), ((5, 33, 896, 64), 0, True, 100)):
         q, k, v = make_inputs(fa, shape, dtype, seed=77)
         tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
         o1, l1 = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, sched=1)
