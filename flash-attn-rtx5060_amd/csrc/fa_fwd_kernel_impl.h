@@ -248,14 +248,15 @@ template <bool BF16> __device__ __forceinline__ f32x2 storage_product2(uint32_t 
     return f32x2{__builtin_bit_cast(float, r << 16), __builtin_bit_cast(float, r & 0xffff0000u)};
 }
 
-// Queries 0..rows-1 of a head (query i at key position i + pos_off, all positions below 32) against keys
-// 0..31.  The 32 x D blocks of Q, K and V are staged in LDS once (K with its 16-byte chunks XOR-swizzled by the
-// row, so that 32 lanes reading one chunk of 32 different rows do not collide), everything else runs from
-// there.  LDS use: 3 * 32 * D * 2 + 2 * 4096 + 128 bytes.
+// Queries row0..row1-1 of a head (query i at key position i + pos_off, all positions below 32) against keys
+// 0..31.  The 32 x D blocks of Q, K and V (the rows needed) are staged in LDS once (K with its 16-byte chunks
+// XOR-swizzled by the row, so that 32 lanes reading one chunk of 32 different rows do not collide), everything
+// else runs from there.  LDS use: 3 * 32 * D * 2 + 2 * 4096 + 128 bytes.
 template <bool BF16, int D>
-__device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
+__device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, const uint16_t *Vh, uint16_t *Oh,
                                     float *o32 /* null, or [rows][D] fp32 to write instead of Oh */,
-                                    float *lse_h, int rows /* queries 0..rows-1 */, int pos_off /* query i sits at key position i + pos_off */,
+                                    float *lse_h, int row0, int row1 /* queries row0..row1-1 */,
+                                    int pos_off /* query i sits at key position i + pos_off */,
                                     int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
                                     uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
@@ -266,25 +267,23 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
     float *sc = reinterpret_cast<float *>(Vs + R * D), *ex = sc + R * R, *rsum = ex + R * R;
     uint32_t *pbits = reinterpret_cast<uint32_t *>(ex);     // after the softmax: p as two copies of its storage bits
     const int tid = threadIdx.x, nthr = blockDim.x;
-    const int nkeys = rows + pos_off;                       // keys 0..nkeys-1 are the ones any of these queries sees
+    const int nrows = row1 - row0;
+    const int nkeys = row1 + pos_off;                       // keys 0..nkeys-1 are the ones any of these queries sees
     for (int idx = tid; idx < R * CPR; idx += nthr) {
         const int row = idx / CPR, c = idx % CPR;
-        u32x4 q4 = {0, 0, 0, 0}, k4 = {0, 0, 0, 0}, v4 = {0, 0, 0, 0};
-        if (row < rows) q4 = *reinterpret_cast<const u32x4 *>(Qh + (size_t)row * q_rs + 8 * c);
+        if (row >= row0 && row < row1)
+            *reinterpret_cast<u32x4 *>(Qs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Qh + (size_t)row * q_rs + 8 * c);
         if (row < nkeys) {
-            k4 = *reinterpret_cast<const u32x4 *>(Kh + (size_t)row * k_rs + 8 * c);
-            v4 = *reinterpret_cast<const u32x4 *>(Vh + (size_t)row * v_rs + 8 * c);
+            *reinterpret_cast<u32x4 *>(Ks + row * D + 8 * (c ^ (row & (CPR - 1)))) = *reinterpret_cast<const u32x4 *>(Kh + (size_t)row * k_rs + 8 * c);
+            *reinterpret_cast<u32x4 *>(Vs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Vh + (size_t)row * v_rs + 8 * c);
         }
-        *reinterpret_cast<u32x4 *>(Qs + row * D + 8 * c) = q4;
-        *reinterpret_cast<u32x4 *>(Ks + row * D + 8 * (c ^ (row & (CPR - 1)))) = k4;
-        *reinterpret_cast<u32x4 *>(Vs + row * D + 8 * c) = v4;
     }
     __syncthreads();
     // scores (main.cu:189-197), masked entries -inf (main.cu:210-229); query i at position p sees keys p-L..p
-    for (int idx = tid; idx < R * R; idx += nthr) {
-        const int i = idx / R, j = idx % R, p = i + pos_off;
+    for (int idx = tid; idx < nrows * R; idx += nthr) {
+        const int i = row0 + idx / R, j = idx % R, p = i + pos_off;
         float s = -INFINITY;
-        if (i < rows && j <= p && p - j <= L) {
+        if (j <= p && p - j <= L) {
             float sum = 0.0f;
             for (int c = 0; c < CPR; ++c) {
                 const u32x4 qa = *reinterpret_cast<const u32x4 *>(Qs + i * D + 8 * c);
@@ -300,57 +299,63 @@ __device__ void faithful_first_rows(const uint16_t *Qh, const uint16_t *Kh, cons
             // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
             if (slope != 0.0f) s = __fsub_rn(s, __fmul_rn(slope, (float)(p - j)));
         }
-        sc[idx] = s;
+        sc[i * R + j] = s;
     }
     __syncthreads();
     // softmax of each row (main.cu:232-252).  The row maximum does not depend on the order it is taken in and
     // the exponentials are independent, so every thread does one element; only the row sum has to add in
     // index order, and one thread per row does that.
-    for (int idx = tid; idx < R * R; idx += nthr) {
-        const int i = idx / R;
+    for (int idx = tid; idx < nrows * R; idx += nthr) {
+        const int i = row0 + idx / R, e = i * R + idx % R;
         const float *row = sc + i * R;
         float mx = -INFINITY;
         for (int j = 0; j < R; ++j) mx = fmaxf(mx, row[j]);
-        ex[idx] = (i < rows && sc[idx] != -INFINITY) ? expf(sc[idx] - mx) : 0.0f;
+        ex[e] = sc[e] != -INFINITY ? expf(sc[e] - mx) : 0.0f;
     }
     __syncthreads();
-    if (tid < rows) {
-        const float *row = ex + tid * R;
+    if (tid < nrows) {
+        const int i = row0 + tid;
+        const float *row = ex + i * R;
         float sum = 0.0f;
         for (int j = 0; j < R; ++j) sum += row[j];          // masked entries are +0: they change no bit of the sum
-        rsum[tid] = sum;
+        rsum[i] = sum;
         if (lse_h != nullptr) {
             float mx = -INFINITY;
-            for (int j = 0; j < R; ++j) mx = fmaxf(mx, sc[tid * R + j]);
-            lse_h[tid] = mx + logf(sum);
+            for (int j = 0; j < R; ++j) mx = fmaxf(mx, sc[i * R + j]);
+            lse_h[i] = mx + logf(sum);
         }
     }
     __syncthreads();
     // p rounded to the storage type (main.cu:259)
-    for (int idx = tid; idx < R * R; idx += nthr) {
-        const int i = idx / R, j = idx % R;
+    for (int idx = tid; idx < nrows * R; idx += nthr) {
+        const int i = row0 + idx / R, j = idx % R, e = i * R + j;
         float pj = 0.0f;
-        if (i < rows && sc[idx] != -INFINITY) {
-            pj = ex[idx] / rsum[i];
+        if (sc[e] != -INFINITY) {
+            pj = ex[e] / rsum[i];
             if (drop_threshold != 0u) {        // keys 0..31: one 32-key block, two Philox blocks per query
                 const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)(i + pos_off), (uint32_t)((j >> 2) & 1));
                 pj = dropout_keep_byte(d, 4 * (j >> 3) + (j & 3), drop_threshold) ? __fmul_rn(pj, drop_scale) : 0.0f;
             }
         }
         const uint32_t bits = f32_to_storage<BF16>(pj);
-        pbits[idx] = bits | (bits << 16);       // (each thread overwrites only the element it has just read)
+        pbits[e] = bits | (bits << 16);         // (each thread overwrites only the element it has just read)
     }
     __syncthreads();
     // weighted sum (main.cu:255-263), keys in ascending order; masked keys have p = 0 and add nothing.  A thread
     // owns two neighbouring output elements of one row.
-    for (int idx = tid; idx < rows * (D / 2); idx += nthr) {
-        const int i = idx / (D / 2), t2 = idx % (D / 2), p = i + pos_off;
+    for (int idx = tid; idx < nrows * (D / 2); idx += nthr) {
+        const int i = row0 + idx / (D / 2), t2 = idx % (D / 2), p = i + pos_off;
         const int lo = p - L > 0 ? p - L : 0;
         float s0 = 0.0f, s1 = 0.0f;
-        for (int j = lo; j <= p; ++j) {
-            const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *reinterpret_cast<const uint32_t *>(Vs + j * D + 2 * t2));
-            s0 += pr[0];
-            s1 += pr[1];
+        // (a fixed trip count with a predicate instead of a loop from lo to p: unrolled, the LDS reads are issued
+        // together instead of one latency after the other; the additions keep their order)
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            if (j >= lo && j <= p) {
+                const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *reinterpret_cast<const uint32_t *>(Vs + j * D + 2 * t2));
+                s0 += pr[0];
+                s1 += pr[1];
+            }
         }
         const uint32_t packed = Num<BF16>::pack2(s0, s1);
         if (o32 != nullptr) {
@@ -390,6 +395,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     constexpr int NF = NPV + NQK;                 // every fragment feeds RB matrix instructions
     constexpr int PD = RB == 1 ? 6 : 3;           // LDS reads run this many fragments ahead
     constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
+    // (the first-rows path works in LDS behind the K stages that the requests for the next item fill)
+    static_assert(NST <= 3 && LA * TILEB + 3 * kFaithfulRows * D * 2 + 2 * 4096 + 128 <= 2 * NST * TILEB, "first-rows path does not fit behind the requested stages");
     constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
     static_assert(INSTR % NW == 0, "tile must divide over the waves");
     static_assert(NST >= 2 && NST <= 4 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
@@ -1014,12 +1021,23 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32
     // (with more queries than keys, pos_off < 0, the path is not taken);
     // fa_fwd_params.exact_first_rows switches the path off)
-    const bool faithful = MASKED && a.R == 0 && q0 == 0 && pos_off >= 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
+    const bool first_rows_on = MASKED && a.R == 0 && pos_off >= 0 && pos_off < kFaithfulRows && split == 0 && pack == 1 && !a.exact_first_rows;
+    const bool faithful = first_rows_on && q0 == 0;         // this item's own rows 0..31 are not stored by the epilogue
     const int f_rows = !faithful ? 0 : !GENERAL ? kFaithfulRows : (kFaithfulRows - pos_off < S ? kFaithfulRows - pos_off : S);
+    // Which of those rows THIS item recomputes.  General layouts: the item with the head's first block, all of
+    // them.  Contiguous layout: the 32 rows are dealt in 2 or 4 parts to the head's first query blocks, one
+    // part each -- under a static schedule the workgroups that run the path are the critical path of a short
+    // problem (c2: 64 of 256 workgroups carried 7.7 us each), and every pair of items of the snake then gets one.
+    int fr0 = 0, fr1 = 0;
+    if (GENERAL) fr1 = f_rows;
+    else if (first_rows_on) {
+        const int parts = a.n_qblocks >= 4 ? 4 : a.n_qblocks >= 2 ? 2 : 1;
+        if (qblock < parts) { fr0 = qblock * (kFaithfulRows / parts); fr1 = fr0 + kFaithfulRows / parts; }
+    }
     // ---- the next work item, and the first requests for it
     const int next_item = take_item(pass + 1, ticket_ahead);
-    // (an item that ends with the first-rows path uses the K stages' LDS for it: nothing is requested then)
-    if (!GENERAL && RB == 1 && next_item >= 0 && !faithful) {
+    // (the first-rows path below works in the LDS behind the K stages that are filled here)
+    if (!GENERAL && RB == 1 && next_item >= 0) {
         int nbh, nqb, nt0, nt1;
         fa_item_decode(next_item, a.BH, a.n_qblocks, a.descending, &nbh, &nqb);
         const size_t noff = (size_t)nbh * S * D;
@@ -1088,10 +1106,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
     }
     FA_TL(5);
-    if (faithful)     // the last iteration ended with a barrier: the LDS stages are free
+    if (fr1 > fr0)    // the last iteration ended with a barrier: the LDS behind the first LA K stages is free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
-                                     f_rows, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
-                                     a.seed_lo, a.seed_hi, (uint32_t)bh, smem);
+                                     fr0, fr1, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
+                                     a.seed_lo, a.seed_hi, (uint32_t)bh, smem + LA * TILEB);
     FA_TL(6);
 #ifdef FA_TIMELINE
     if (tid == 0 && g_fa_timeline != nullptr) {
