@@ -260,22 +260,27 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
                                     int L, float scale, float slope,
                                     int q_rs, int k_rs, int v_rs, int o_rs /* row strides in elements */,
                                     uint32_t drop_threshold, float drop_scale, uint32_t seed_lo, uint32_t seed_hi, uint32_t bh,
-                                    char *lds)
+                                    uint32_t lds /* LDS byte address of the work area */)
 {
     constexpr int R = kFaithfulRows, CPR = D / 8;
-    uint16_t *Qs = reinterpret_cast<uint16_t *>(lds), *Ks = Qs + R * D, *Vs = Ks + R * D;
-    float *sc = reinterpret_cast<float *>(Vs + R * D), *ex = sc + R * R, *rsum = ex + R * R;
-    uint32_t *pbits = reinterpret_cast<uint32_t *>(ex);     // after the softmax: p as two copies of its storage bits
+    // (LDS-typed pointers: through generic ones every access would be a flat instruction)
+    typedef __attribute__((address_space(3))) uint16_t lds_u16;
+    typedef __attribute__((address_space(3))) float lds_f32;
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+    lds_u16 *Qs = (lds_u16 *)(uintptr_t)lds, *Ks = Qs + R * D, *Vs = Ks + R * D;
+    lds_f32 *sc = (lds_f32 *)(Vs + R * D), *ex = sc + R * R, *rsum = ex + R * R;
+    lds_u32 *pbits = (lds_u32 *)ex;                         // after the softmax: p as two copies of its storage bits
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int nrows = row1 - row0;
     const int nkeys = row1 + pos_off;                       // keys 0..nkeys-1 are the ones any of these queries sees
     for (int idx = tid; idx < R * CPR; idx += nthr) {
         const int row = idx / CPR, c = idx % CPR;
         if (row >= row0 && row < row1)
-            *reinterpret_cast<u32x4 *>(Qs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Qh + (size_t)row * q_rs + 8 * c);
+            *(lds_u32x4 *)(Qs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Qh + (size_t)row * q_rs + 8 * c);
         if (row < nkeys) {
-            *reinterpret_cast<u32x4 *>(Ks + row * D + 8 * (c ^ (row & (CPR - 1)))) = *reinterpret_cast<const u32x4 *>(Kh + (size_t)row * k_rs + 8 * c);
-            *reinterpret_cast<u32x4 *>(Vs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Vh + (size_t)row * v_rs + 8 * c);
+            *(lds_u32x4 *)(Ks + row * D + 8 * (c ^ (row & (CPR - 1)))) = *reinterpret_cast<const u32x4 *>(Kh + (size_t)row * k_rs + 8 * c);
+            *(lds_u32x4 *)(Vs + row * D + 8 * c) = *reinterpret_cast<const u32x4 *>(Vh + (size_t)row * v_rs + 8 * c);
         }
     }
     __syncthreads();
@@ -286,8 +291,8 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
         if (j <= p && p - j <= L) {
             float sum = 0.0f;
             for (int c = 0; c < CPR; ++c) {
-                const u32x4 qa = *reinterpret_cast<const u32x4 *>(Qs + i * D + 8 * c);
-                const u32x4 kb = *reinterpret_cast<const u32x4 *>(Ks + j * D + 8 * (c ^ (j & (CPR - 1))));
+                const u32x4 qa = *(const lds_u32x4 *)(Qs + i * D + 8 * c);
+                const u32x4 kb = *(const lds_u32x4 *)(Ks + j * D + 8 * (c ^ (j & (CPR - 1))));
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     const f32x2 pr = storage_product2<BF16>(qa[w], kb[w]);
@@ -307,20 +312,23 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
     // index order, and one thread per row does that.
     for (int idx = tid; idx < nrows * R; idx += nthr) {
         const int i = row0 + idx / R, e = i * R + idx % R;
-        const float *row = sc + i * R;
+        const lds_f32 *row = sc + i * R;
         float mx = -INFINITY;
+#pragma unroll
         for (int j = 0; j < R; ++j) mx = fmaxf(mx, row[j]);
         ex[e] = sc[e] != -INFINITY ? expf(sc[e] - mx) : 0.0f;
     }
     __syncthreads();
     if (tid < nrows) {
         const int i = row0 + tid;
-        const float *row = ex + i * R;
+        const lds_f32 *row = ex + i * R;
         float sum = 0.0f;
+#pragma unroll
         for (int j = 0; j < R; ++j) sum += row[j];          // masked entries are +0: they change no bit of the sum
         rsum[i] = sum;
         if (lse_h != nullptr) {
             float mx = -INFINITY;
+#pragma unroll
             for (int j = 0; j < R; ++j) mx = fmaxf(mx, sc[i * R + j]);
             lse_h[i] = mx + logf(sum);
         }
@@ -351,8 +359,9 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
         // together instead of one latency after the other; the additions keep their order)
 #pragma unroll
         for (int j = 0; j < R; ++j) {
+            if (j >= nkeys) break;              // (uniform: no query of this call sees a later key)
             if (j >= lo && j <= p) {
-                const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *reinterpret_cast<const uint32_t *>(Vs + j * D + 2 * t2));
+                const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *(const lds_u32 *)(Vs + j * D + 2 * t2));
                 s0 += pr[0];
                 s1 += pr[1];
             }
@@ -1109,7 +1118,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     if (fr1 > fr0)    // the last iteration ended with a barrier: the LDS behind the first LA K stages is free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      fr0, fr1, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
-                                     a.seed_lo, a.seed_hi, (uint32_t)bh, smem + LA * TILEB);
+                                     a.seed_lo, a.seed_hi, (uint32_t)bh, lds0 + LA * TILEB);
     FA_TL(6);
 #ifdef FA_TIMELINE
     if (tid == 0 && g_fa_timeline != nullptr) {
