@@ -290,15 +290,23 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
         float s = -INFINITY;
         if (j <= p && p - j <= L) {
             float sum = 0.0f;
-            for (int c = 0; c < CPR; ++c) {
-                const u32x4 qa = *(const lds_u32x4 *)(Qs + i * D + 8 * c);
-                const u32x4 kb = *(const lds_u32x4 *)(Ks + j * D + 8 * (c ^ (j & (CPR - 1))));
+            // (the operands are read four chunks at a time, ahead of the additions that have to wait for each other)
 #pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const f32x2 pr = storage_product2<BF16>(qa[w], kb[w]);
-                    sum += pr[0];
-                    sum += pr[1];
+            for (int c0 = 0; c0 < CPR; c0 += 4) {
+                u32x4 qa[4], kb[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    qa[c] = *(const lds_u32x4 *)(Qs + i * D + 8 * (c0 + c));
+                    kb[c] = *(const lds_u32x4 *)(Ks + j * D + 8 * ((c0 + c) ^ (j & (CPR - 1))));
                 }
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const f32x2 pr = storage_product2<BF16>(qa[c][w], kb[c][w]);
+                        sum += pr[0];
+                        sum += pr[1];
+                    }
             }
             s = sum * scale;
             // ALiBi as the verifier applies it (main.cu:200-207): a rounded product, then a rounded difference
@@ -355,13 +363,19 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
         const int i = row0 + idx / (D / 2), t2 = idx % (D / 2), p = i + pos_off;
         const int lo = p - L > 0 ? p - L : 0;
         float s0 = 0.0f, s1 = 0.0f;
-        // (a fixed trip count with a predicate instead of a loop from lo to p: unrolled, the LDS reads are issued
-        // together instead of one latency after the other; the additions keep their order)
+        // (all operands are read first, with a fixed trip count, and the additions follow in key order under a
+        // predicate: read one by one inside a loop from lo to p, every step waited for its own LDS round trip,
+        // 85 ns per key)
+        uint32_t pw[R], vw[R];
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            if (j >= nkeys) break;              // (uniform: no query of this call sees a later key)
+            pw[j] = pbits[i * R + j];
+            vw[j] = *(const lds_u32 *)(Vs + j * D + 2 * t2);        // (rows past the last key hold stale bytes: never used)
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
             if (j >= lo && j <= p) {
-                const f32x2 pr = storage_product2<BF16>(pbits[i * R + j], *(const lds_u32 *)(Vs + j * D + 2 * t2));
+                const f32x2 pr = storage_product2<BF16>(pw[j], vw[j]);
                 s0 += pr[0];
                 s1 += pr[1];
             }
