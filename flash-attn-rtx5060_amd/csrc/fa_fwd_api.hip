@@ -22,6 +22,8 @@
 
 hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                         hipStream_t stream);
+hipError_t fa_launch_forward_strided(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
+                                     hipStream_t stream);
 hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
@@ -302,6 +304,7 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     a.lse_part = a.o_part != nullptr ? a.o_part + (size_t)a.n_splits * p->B * p->N * p->S * p->d : nullptr;
     a.pack = packed_group(p);
     bool general = a.Hk != p->N || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
+    bool strided = false;       // the regular problem, not stored contiguous [B,N,S,d]
     {
         const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
         long long eff[4][3];
@@ -313,7 +316,7 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
             const bool given = st[0] != 0 || st[1] != 0 || st[2] != 0;
             for (int k = 0; k < 3; ++k) {
                 eff[t][k] = given ? st[k] : dense[k];
-                if (eff[t][k] != dense[k]) general = true;
+                if (eff[t][k] != dense[k]) strided = true;
             }
         }
         a.q_bs = eff[0][0]; a.q_hs = eff[0][1]; a.q_rs = (int)eff[0][2];
@@ -357,7 +360,8 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
     a.seed_hi = (unsigned)(p->seed >> 32);
     a.exact_first_rows = p->exact_first_rows != 0;
-    hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general : fa_launch_forward_contiguous)(
+    hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general
+                    : strided ? fa_launch_forward_strided : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
     if (a.n_splits > 1) {

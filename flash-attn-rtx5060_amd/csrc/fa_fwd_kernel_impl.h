@@ -401,7 +401,7 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>
 __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
 {
     constexpr int WR = 32 * RB;                   // query rows per wave
@@ -550,11 +550,20 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         Vh = a.V + (size_t)bi * a.v_bs + (size_t)hk * a.v_hs;
         Oh = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs;
     } else {
+        if (STRIDED) {
+        const int bi = bh / a.H, hi = bh - bi * a.H;
+        Qh = a.Q + (size_t)bi * a.q_bs + (size_t)hi * a.q_hs;
+        Kh = a.K + (size_t)bi * a.k_bs + (size_t)hi * a.k_hs;
+        Vh = a.V + (size_t)bi * a.v_bs + (size_t)hi * a.v_hs;
+        Oh = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs;
+        } else {
         const size_t head_off = (size_t)bh * S * D;
         Qh = a.Q + head_off; Kh = a.K + head_off; Vh = a.V + head_off;
         Oh = a.O + head_off;
+        }
     }
-    const int q_rs = GENERAL ? a.q_rs : D, k_rs = GENERAL ? a.k_rs : D, v_rs = GENERAL ? a.v_rs : D, o_rs = GENERAL ? a.o_rs : D;
+    const int q_rs = (GENERAL || STRIDED) ? a.q_rs : D, k_rs = (GENERAL || STRIDED) ? a.k_rs : D, v_rs = (GENERAL || STRIDED) ? a.v_rs : D,
+              o_rs = (GENERAL || STRIDED) ? a.o_rs : D;
 
     const int q0 = qblock * BR;
     const int qw = q0 + wave * WR;          // first query row of this wave
@@ -1063,20 +1072,29 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     if (!GENERAL && RB == 1 && next_item >= 0) {
         int nbh, nqb, nt0, nt1;
         fa_item_decode(next_item, a.BH, a.n_qblocks, a.descending, &nbh, &nqb);
-        const size_t noff = (size_t)nbh * S * D;
+        const uint16_t *nQ, *nK, *nV;
+        if (STRIDED) {
+            const int nbi = nbh / a.H, nhi = nbh - nbi * a.H;
+            nQ = a.Q + (size_t)nbi * a.q_bs + (size_t)nhi * a.q_hs;
+            nK = a.K + (size_t)nbi * a.k_bs + (size_t)nhi * a.k_hs;
+            nV = a.V + (size_t)nbi * a.v_bs + (size_t)nhi * a.v_hs;
+        } else {
+            const size_t noff = (size_t)nbh * S * D;
+            nQ = a.Q + noff; nK = a.K + noff; nV = a.V + noff;
+        }
         const int nq0 = nqb * BR;
         fa_tile_range(S, kBlockKeys, a.L, a.R, nq0, S - nq0 < BR ? S - nq0 : BR, &nt0, &nt1);
         // (every LDS stage is free: the last iteration ended with a barrier)
-        issue_k_from(a.K + noff, nt0, 0);
-        if (LA > 1 && nt0 + 1 <= nt1) issue_k_from(a.K + noff, nt0 + 1, 1);
-        if (LA > 2 && nt0 + 2 <= nt1) issue_k_from(a.K + noff, nt0 + 2, 2);
-        if (LA > 2) issue_v_from(a.V + noff, nt0, 0);
+        issue_k_from(nK, nt0, 0);
+        if (LA > 1 && nt0 + 1 <= nt1) issue_k_from(nK, nt0 + 1, 1);
+        if (LA > 2 && nt0 + 2 <= nt1) issue_k_from(nK, nt0 + 2, 2);
+        if (LA > 2) issue_v_from(nV, nt0, 0);
         // (S is a multiple of 128: a wave has all its rows or none; one without rows never uses its fragments and
         // reads those of the block's first wave, so that no select has to wait for the data)
         const int nrow = nq0 + (nq0 + wave * WR < S ? wave * WR : 0) + l32;
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-            qf[0][s] = *reinterpret_cast<const u32x4 *>(a.Q + noff + (size_t)nrow * D + 16 * s + 8 * half);
+            qf[0][s] = *reinterpret_cast<const u32x4 *>(nQ + (size_t)nrow * q_rs + 16 * s + 8 * half);
         next_requested = true;
     }
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
@@ -1189,7 +1207,7 @@ __global__ void __launch_bounds__(256) fa_combine_splits(const FaKernelArgs a)
     if (a.lse != nullptr && c4 == 0) a.lse[row] = mx == -INFINITY ? -INFINITY : mx + __logf(wsum);
 }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>
 hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
@@ -1198,7 +1216,7 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 #else
     const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the two words of the queue schedule
 #endif
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST>;
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST, STRIDED>;
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
     const unsigned long long dev_bit = 1ull << fa_launch_device();
@@ -1234,15 +1252,15 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 #else
 #define FA_ROWS64_CASE(BF, DD, MK, AL)
 #endif
-template <bool GENERAL, bool DROPOUT>
+template <bool GENERAL, bool DROPOUT, bool STRIDED = false>
 hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
         FA_ROWS64_CASE(BF, DD, MK, AL) \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? FA_NST8_GENERAL : FA_NST8)>(a, grid, stream); \
-        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? FA_NST8_GENERAL : FA_NST8), STRIDED>(a, grid, stream); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2, STRIDED>(a, grid, stream); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
     FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)

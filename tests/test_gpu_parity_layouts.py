@@ -151,3 +151,29 @@ def test_general_layouts_under_every_schedule(fa, oracle, shape, Hk, S_real):
         outs.append((o, lse))
     for o, lse in outs[1:]:
         assert torch.equal(o.view(torch.int16), outs[0][0].view(torch.int16)) and torch.equal(lse, outs[0][1])
+
+
+@pytest.mark.parametrize("shape,dtype,causal,wl,sched", [((2, 8, 1024, 128), 0, True, -1, 0), ((8, 40, 384, 64), 1, True, 100, 2),
+                                                         ((4, 16, 2176, 128), 0, False, -1, 3), ((1, 4, 256, 64), 0, False, -1, 1)])
+def test_regular_problem_in_strided_layouts_matches_the_contiguous_run_bit_for_bit(fa, shape, dtype, causal, wl, sched):
+    """Lengths a multiple of 128, one K/V head per query head: a strided layout ([B,S,H,D] views, rows padded to a
+    larger stride, an output with its own layout) runs the contiguous kernels' instruction stream with strides from
+    the arguments, so the bits must be those of the contiguous run (several passes over the resident grid included:
+    what a workgroup requests ahead for its next item is addressed through the same strides)."""
+    import torch
+    B, H, S, D = shape
+    q, k, v = make_inputs(fa, shape, dtype, seed=91)
+    tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    o_ref, lse_ref = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, sched=sched)
+    # [B,S,H,D] storage
+    sq, sk, sv = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv))
+    out = torch.full((B, S, H, D), float("nan"), dtype=tq.dtype, device="cuda").transpose(1, 2)
+    o1, lse1 = fa.flash_attention_forward(sq, sk, sv, causal=causal, window_left=wl, sched=sched, out=out)
+    # rows padded to D + 64 elements, K and V sharing one buffer
+    pad = torch.zeros((B, H, S, 2 * D + 64), dtype=tq.dtype, device="cuda")
+    pad[..., :D] = tk
+    pad[..., D + 64:] = tv
+    o2, lse2 = fa.flash_attention_forward(tq, pad[..., :D], pad[..., D + 64:], causal=causal, window_left=wl, sched=sched)
+    torch.cuda.synchronize()
+    for o, lse in ((o1, lse1), (o2, lse2)):
+        assert torch.equal(o.contiguous().view(torch.int16), o_ref.view(torch.int16)) and torch.equal(lse, lse_ref)
