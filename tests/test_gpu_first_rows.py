@@ -25,12 +25,17 @@ def ulp(x, dtype):
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
-@pytest.mark.parametrize("shape,wl,seed", [((2, 4, 256, 128), -1, 29), ((1, 8, 384, 64), -1, 7), ((1, 4, 256, 128), 9, 3),
-                                           ((2, 32, 1024, 128), -1, 29)])
-def test_first_rows_are_the_verifiers_bits(fa, oracle, dtype, shape, wl, seed):
+@pytest.mark.parametrize("shape,wl,seed,sched", [((2, 4, 256, 128), -1, 29, 0), ((1, 8, 384, 64), -1, 7, 0), ((1, 4, 256, 128), 9, 3, 0),
+                                                 ((2, 32, 1024, 128), -1, 29, 0),
+                                                 # the path dealt in one, two and four parts, in workgroups of 128 and of 256
+                                                 # rows, under every schedule (several passes over the resident grid included)
+                                                 ((1, 4, 128, 64), -1, 5, 0), ((1, 4, 512, 128), -1, 6, 2), ((4, 64, 2048, 64), -1, 28, 0),
+                                                 ((4, 64, 2048, 64), 40, 28, 3), ((8, 80, 768, 128), -1, 9, 2), ((8, 80, 512, 64), -1, 10, 3),
+                                                 ((8, 80, 256, 64), -1, 11, 1)])
+def test_first_rows_are_the_verifiers_bits(fa, oracle, dtype, shape, wl, seed, sched):
     B, H, S, D = shape
     q, k, v = make_inputs(fa, shape, dtype, seed)
-    o, lse = fa.flash_attention_forward(to_torch(q, dtype), to_torch(k, dtype), to_torch(v, dtype), causal=True, window_left=wl)
+    o, lse = fa.flash_attention_forward(to_torch(q, dtype), to_torch(k, dtype), to_torch(v, dtype), causal=True, window_left=wl, sched=sched)
     rows = np.array([bh * S + r for bh in range(B * H) for r in range(32)], dtype=np.int64)
     o_ref, lse_ref = oracle.rows(q, k, v, rows, dtype, None, True, wl, -1)
     got = from_torch(o).reshape(-1, D)[rows]
