@@ -539,7 +539,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             }
         }
     }
-    if (row_ok) {
+    // (the lane's row and column offset are derived again here, from the hardware's lane index and tied to this
+    // place: taken from the values computed at the top, the compiler forms the store addresses there and keeps
+    // them in registers, or in scratch memory, through the whole loop)
+    int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(lane_e));
+    const int key_e = kw + (lane_e & 31), half_e = lane_e >> 5;
+    if (active && key_e < Sk) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -549,8 +555,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
                 wk[1] = N::pack2(dk[db][4 * g + 2] * a.scale, dk[db][4 * g + 3] * a.scale);
                 wv[0] = N::pack2(dv[db][4 * g], dv[db][4 * g + 1]);
                 wv[1] = N::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
-                *reinterpret_cast<u32x2 *>(dKh + (size_t)my_kc * dk_rs + 32 * db + 8 * g + 4 * half) = wk;
-                *reinterpret_cast<u32x2 *>(dVh + (size_t)my_kc * dv_rs + 32 * db + 8 * g + 4 * half) = wv;
+                *reinterpret_cast<u32x2 *>(dKh + (size_t)key_e * dk_rs + 32 * db + 8 * g + 4 * half_e) = wk;
+                *reinterpret_cast<u32x2 *>(dVh + (size_t)key_e * dv_rs + 32 * db + 8 * g + 4 * half_e) = wv;
             }
     }
 }
