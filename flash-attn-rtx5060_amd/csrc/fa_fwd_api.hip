@@ -48,20 +48,32 @@ int waves_for(int B, int N, int S)
 
 thread_local char g_last_error[256] = "";
 
-std::atomic<unsigned> g_eager_ticket{0}, g_capture_ticket{0};
+std::atomic<unsigned> g_capture_ticket{0};
+// eager launches: which stream owns which counter set of a device (0 = free; the legacy default stream is kept as 1)
+std::atomic<uintptr_t> g_slot_owner[kFaMaxDevices][kFaQueueSlots / 2];
 
-// A counter set for one FA_SCHED_QUEUE launch.  A launch that is being captured into a graph keeps its set for
-// every replay of that graph, so captured launches take their sets from the upper half of the table and eager
-// launches from the lower half: a replaying graph never shares counters with eager work on another stream.
-// Within a half the sets go round-robin.
+// A counter set for one FA_SCHED_QUEUE launch, or null when none can be given safely (the caller then walks the
+// list with the fixed snake).  Eager launches: a set belongs to a stream -- launches on one stream run one after
+// the other, so they may share it, and every launch leaves it rewound; a device hands out sixteen sets, to the
+// first sixteen streams that ask (a stream keeps its set for the life of the process), and further streams get
+// none.  A launch that is being captured into a graph keeps its set for every replay of that graph, and a replay
+// may run next to anything, so captured launches take their sets round-robin from the other sixteen: a replaying
+// graph never shares counters with eager work, and up to sixteen captured launches never with each other.
 unsigned *work_queue_for_launch(const FaDeviceState *ds, hipStream_t stream)
 {
     constexpr unsigned half = (unsigned)kFaQueueSlots / 2u;
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
     const bool capturing = stream != nullptr && hipStreamIsCapturing(stream, &status) == hipSuccess &&
                            status == hipStreamCaptureStatusActive;
-    const unsigned slot = capturing ? half + g_capture_ticket.fetch_add(1u) % half : g_eager_ticket.fetch_add(1u) % half;
-    return ds->queues + 16u * slot;
+    if (capturing) return ds->queues + 16u * (half + g_capture_ticket.fetch_add(1u) % half);
+    const uintptr_t key = stream == nullptr ? (uintptr_t)1 : reinterpret_cast<uintptr_t>(stream);
+    std::atomic<uintptr_t> *owners = g_slot_owner[fa_launch_device()];
+    for (unsigned i = 0; i < half; ++i) {
+        uintptr_t seen = owners[i].load(std::memory_order_acquire);
+        if (seen == 0 && owners[i].compare_exchange_strong(seen, key, std::memory_order_acq_rel)) seen = key;
+        if (seen == key) return ds->queues + 16u * i;
+    }
+    return nullptr;
 }
 
 int device_fail(hipError_t e, const char *what)
@@ -411,7 +423,10 @@ int fa_reset_work_queues(void)
     e = hipDeviceSynchronize();
     if (e != hipSuccess) return device_fail(e, "synchronize");
     e = hipMemset(ds->queues, 0, (size_t)kFaQueueSlots * 16 * sizeof(unsigned));
-    return e == hipSuccess ? FA_OK : device_fail(e, "work queue reset");
+    if (e != hipSuccess) return device_fail(e, "work queue reset");
+    // (nothing is in flight after the synchronisation: streams may claim their sets anew)
+    for (int i = 0; i < kFaQueueSlots / 2; ++i) g_slot_owner[fa_launch_device()][i].store(0, std::memory_order_release);
+    return FA_OK;
 }
 
 int run_flash_attention(int B, int N, int S, int d, void *Q, void *K, void *V, void *O, void *L, void *M,

@@ -135,3 +135,27 @@ def test_schedules_agree_bitwise(fa):
             fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, sched=3, out=o3, lse=l3)
         torch.cuda.synchronize()
         assert torch.equal(o1.view(torch.int16), o3.view(torch.int16)) and torch.equal(l1, l3)
+
+
+def test_queue_schedule_on_many_streams_at_once(fa):
+    """Twenty-four streams launch the queue schedule concurrently, several times each: the first sixteen streams
+    own a counter set each, the others fall back to the fixed work order; every output must be the reference's
+    bits (two launches sharing counters would skip or repeat work items)."""
+    import torch
+    shape, dtype = (2, 16, 2048, 128), 0
+    q, k, v = make_inputs(fa, shape, dtype, seed=93)
+    tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    o_ref, l_ref = fa.flash_attention_forward(tq, tk, tv, causal=True, sched=1)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(24)]
+    outs = []
+    for rep in range(3):
+        for s in streams:
+            with torch.cuda.stream(s):
+                o = torch.full_like(o_ref, float("nan"))
+                l = torch.full_like(l_ref, float("nan"))
+                fa.flash_attention_forward(tq, tk, tv, causal=True, sched=3, out=o, lse=l)
+                outs.append((o, l))
+    torch.cuda.synchronize()
+    for o, l in outs:
+        assert torch.equal(o.view(torch.int16), o_ref.view(torch.int16)) and torch.equal(l, l_ref)
