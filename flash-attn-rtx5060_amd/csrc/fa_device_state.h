@@ -6,7 +6,8 @@
 #include <hip/hip_runtime.h>
 
 constexpr int kFaMaxDevices = 64;
-constexpr int kFaQueueSlots = 32;                              // work-queue counter sets per device
+constexpr int kFaEagerQueueSlots = 16;                         // counter sets for eager launches, one per stream
+constexpr int kFaQueueSlots = 256;                             // work-queue counter sets per device; the rest serve captured launches
 constexpr unsigned long long kFaStaticScratchBytes = 32ull << 20;   // key-split scratch per device
 
 struct FaDeviceState {

@@ -48,27 +48,31 @@ int waves_for(int B, int N, int S)
 
 thread_local char g_last_error[256] = "";
 
-std::atomic<unsigned> g_capture_ticket{0};
+std::atomic<unsigned> g_capture_ticket[kFaMaxDevices];     // captured queue launches so far, per device
 // eager launches: which stream owns which counter set of a device (0 = free; the legacy default stream is kept as 1)
-std::atomic<uintptr_t> g_slot_owner[kFaMaxDevices][kFaQueueSlots / 2];
+std::atomic<uintptr_t> g_slot_owner[kFaMaxDevices][kFaEagerQueueSlots];
 
 // A counter set for one FA_SCHED_QUEUE launch, or null when none can be given safely (the caller then walks the
 // list with the fixed snake).  Eager launches: a set belongs to a stream -- launches on one stream run one after
 // the other, so they may share it, and every launch leaves it rewound; a device hands out sixteen sets, to the
 // first sixteen streams that ask (a stream keeps its set for the life of the process), and further streams get
 // none.  A launch that is being captured into a graph keeps its set for every replay of that graph, and a replay
-// may run next to anything, so captured launches take their sets round-robin from the other sixteen: a replaying
-// graph never shares counters with eager work, and up to sixteen captured launches never with each other.
+// may run next to anything: every captured launch gets a set of its own from the remaining 240, for good, and
+// when those are used up captured launches get none.  No two launches that can run at the same time ever share
+// counters.
 unsigned *work_queue_for_launch(const FaDeviceState *ds, hipStream_t stream)
 {
-    constexpr unsigned half = (unsigned)kFaQueueSlots / 2u;
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
     const bool capturing = stream != nullptr && hipStreamIsCapturing(stream, &status) == hipSuccess &&
                            status == hipStreamCaptureStatusActive;
-    if (capturing) return ds->queues + 16u * (half + g_capture_ticket.fetch_add(1u) % half);
+    if (capturing) {
+        const unsigned n = g_capture_ticket[fa_launch_device()].fetch_add(1u, std::memory_order_relaxed);
+        if (n >= (unsigned)(kFaQueueSlots - kFaEagerQueueSlots)) return nullptr;
+        return ds->queues + 16u * ((unsigned)kFaEagerQueueSlots + n);
+    }
     const uintptr_t key = stream == nullptr ? (uintptr_t)1 : reinterpret_cast<uintptr_t>(stream);
     std::atomic<uintptr_t> *owners = g_slot_owner[fa_launch_device()];
-    for (unsigned i = 0; i < half; ++i) {
+    for (unsigned i = 0; i < (unsigned)kFaEagerQueueSlots; ++i) {
         uintptr_t seen = owners[i].load(std::memory_order_acquire);
         if (seen == 0 && owners[i].compare_exchange_strong(seen, key, std::memory_order_acq_rel)) seen = key;
         if (seen == key) return ds->queues + 16u * i;
@@ -425,7 +429,7 @@ int fa_reset_work_queues(void)
     e = hipMemset(ds->queues, 0, (size_t)kFaQueueSlots * 16 * sizeof(unsigned));
     if (e != hipSuccess) return device_fail(e, "work queue reset");
     // (nothing is in flight after the synchronisation: streams may claim their sets anew)
-    for (int i = 0; i < kFaQueueSlots / 2; ++i) g_slot_owner[fa_launch_device()][i].store(0, std::memory_order_release);
+    for (int i = 0; i < kFaEagerQueueSlots; ++i) g_slot_owner[fa_launch_device()][i].store(0, std::memory_order_release);
     return FA_OK;
 }
 

@@ -6,8 +6,9 @@
 #include <mutex>
 
 // Work queues of FA_SCHED_QUEUE launches: kFaQueueSlots sets of nine counters, all zero between launches (the
-// last workgroup of a launch rewinds its set).  Launches take the sets round-robin, so launches that overlap
-// on one device do not share a set unless more than half of kFaQueueSlots of them are in flight at once.
+// last workgroup of a launch rewinds its set).  Which launch gets which set is the launcher's business
+// (work_queue_for_launch in fa_fwd_api.hip): a set per stream for eager launches, a set of its own for every
+// captured launch.
 static __device__ __align__(256) unsigned g_work_queues[kFaQueueSlots][16];
 
 // Scratch of fa_fwd_split_static: the fp32 partial outputs and logsumexps of a launch with key splits, for

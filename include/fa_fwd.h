@@ -153,16 +153,15 @@ int fa_fwd(const fa_fwd_params *p, void *stream);
 int fa_fwd_split_static(const fa_fwd_params *p, void *stream);
 unsigned long long fa_fwd_static_scratch_bytes(void);
 
-/* FA_SCHED_QUEUE keeps its counters in the library's own device memory: 32 sets per device; the last workgroup
+/* FA_SCHED_QUEUE keeps its counters in the library's own device memory: 256 sets per device; the last workgroup
  * of a launch rewinds its set.  Eager launches: a set belongs to a stream (launches on one stream run one after
  * the other and may share it); the first 16 streams that launch on a device get one each and keep it for the life
  * of the process, launches on further streams walk the work list with FA_SCHED_PERSISTENT's fixed order instead
- * (same results, no counters).  Launches captured into graphs take the other 16 sets round-robin; restriction:
- * graphs captured more than 16 queue launches apart that replay concurrently share a set and give wrong
- * results -- give such launches FA_SCHED_PERSISTENT or FA_SCHED_DISPATCH.  A launch that was killed half-way
- * (device reset, process signal) leaves its set dirty: fa_reset_work_queues() waits for the device, zeroes all
- * sets of the current device and forgets which stream owned which.  Never call it while launches are being
- * captured. */
+ * (same results, no counters).  Every launch captured into a graph gets a set of its own, for good (a replay may
+ * run next to anything): 240 per device and process, after which captured launches use the fixed order as well.
+ * No two launches that can run at the same time share counters.  A launch that was killed half-way (device
+ * reset, process signal) leaves its set dirty: fa_reset_work_queues() waits for the device, zeroes all sets of
+ * the current device and forgets which stream owned which.  Never call it while launches are being captured. */
 int fa_reset_work_queues(void);
 
 /*

@@ -40,3 +40,33 @@ def test_forward_and_backward_replayed_from_a_graph(fa, shape, sched):
         for a, b in zip(got, want):
             assert torch.equal(a.view(torch.int32 if a.dtype == torch.float32 else torch.int16),
                                b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)), (replay, shape, sched)
+
+
+def test_more_captured_queue_launches_than_counter_sets(fa):
+    """Every captured queue launch owns a counter set; a device has 240 of them for captured launches, further ones
+    walk the fixed order.  300 launches captured into one graph, replayed three times on new inputs: every launch's
+    output must be the eager result's bits."""
+    import torch
+    shape = (1, 8, 1024, 64)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = (torch.randn(shape, device="cuda", generator=g).half() for _ in range(3))
+    outs = [torch.empty_like(q) for _ in range(300)]
+    lse = torch.empty(shape[:3], dtype=torch.float32, device="cuda")
+    fa.flash_attention_forward(q, k, v, causal=True, out=outs[0], lse=lse, sched=3)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for o in outs:
+                fa.flash_attention_forward(q, k, v, causal=True, out=o, lse=lse, sched=3)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for t in (q, k, v):
+            t.copy_(torch.randn(shape, device="cuda", generator=g).half())
+        graph.replay()
+        torch.cuda.synchronize()
+        want, _ = fa.flash_attention_forward(q, k, v, causal=True, sched=1)
+        torch.cuda.synchronize()
+        for o in outs:
+            assert torch.equal(o.view(torch.int16), want.view(torch.int16)), replay
