@@ -361,10 +361,15 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     // FA_SCHED_AUTO: with at most one item per resident workgroup there is nothing to schedule (and the
     // queue's counter round trips, 2.3 us each, would double the run time of a 7 us problem); with at most
     // two, the fixed snake pairs every long item with a short one; beyond that the work queue balances best.
-    // Measured: c1 9.5 / 9.5 / 5.8 TFLOP/s (dispatch / snake / queue), c2 431 / 516 / 434, c3 995 / - / 1012.
+    // Measured: c1 9.5 / 9.5 / 5.8 TFLOP/s (dispatch / snake / queue), c2 431 / 611 / 448, c3 995 / 955 / 1030.
     int sched = p->sched;
-    if (sched == FA_SCHED_AUTO)
-        sched = a.n_items <= resident ? FA_SCHED_DISPATCH : a.n_items <= 2 * resident ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
+    // Items that are all alike (no mask, or a window of at most half the length: all but the first few query blocks
+    // of a head see the same number of tiles) need no balancing either, and the fixed order saves them the
+    // counters' barriers: c4 766 against 748 TFLOP/s, c3's shape without a mask 1101 against 1096.
+    if (sched == FA_SCHED_AUTO) {
+        const bool alike = !a.descending || 2LL * a.L <= (long long)p->S;
+        sched = a.n_items <= resident ? FA_SCHED_DISPATCH : (a.n_items <= 2 * resident || alike) ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
+    }
     if (sched == FA_SCHED_PERSISTENT || sched == FA_SCHED_QUEUE) {
         if (grid > resident) grid = resident;
         if (sched == FA_SCHED_QUEUE) a.queue = work_queue_for_launch(ds, static_cast<hipStream_t>(stream));
