@@ -419,6 +419,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     constexpr int PD = RB == 1 ? 6 : 3;           // LDS reads run this many fragments ahead
     constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
     // (the first-rows path works in LDS behind the K stages that the requests for the next item fill)
+    static_assert(GENERAL || LA * TILEB + NW * 32 * ROWB <= 2 * NST * TILEB, "the epilogue's row blocks do not fit behind the requested stages");
     static_assert(NST <= 3 && LA * TILEB + 3 * kFaithfulRows * D * 2 + 2 * 4096 + 128 <= 2 * NST * TILEB, "first-rows path does not fit behind the requested stages");
     constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
     static_assert(INSTR % NW == 0, "tile must divide over the waves");
@@ -1133,6 +1134,41 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                 if (half == 0) lse_part[q] = lse_row;
                 continue;
             }
+            if (!GENERAL && RB == 1) {
+                // Through LDS, so that every store instruction writes whole rows: a lane holds 8-byte pieces of ONE
+                // row, and stored from the registers an instruction touches 32 rows with 16 bytes each (the
+                // address path takes as long for it as for 32 full cache lines); row-major, four (eight) rows of
+                // 256 (128) bytes per instruction.  The wave's 32 x D block sits in LDS that nothing else uses at
+                // this point (behind the K stages that the requests for the next item fill), 16-byte chunks
+                // XOR-swizzled by the row; written and read by this wave only, whose LDS operations complete in order.
+                typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
+                typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+                // (the lane index is taken from the hardware here and tied to this place: derived from threadIdx.x,
+                // these addresses are formed at the top of the kernel and kept in registers through the tile loop)
+                int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+                asm volatile("" : "+v"(lane_e));
+                const int l32_e = lane_e & 31, half_e = lane_e >> 5;
+                const uint32_t obase = lds0 + LA * TILEB + wave * (32 * ROWB);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        u32x2 w;
+                        w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
+                        w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
+                        const int chunk = 4 * db + g;           // 16-byte chunk of the row: elements 8 * chunk .. + 7
+                        *(lds_u32x2 *)(uintptr_t)(obase + l32_e * ROWB + ((chunk ^ (l32_e & (CPR - 1))) << 4) + 8 * half_e) = w;
+                    }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                constexpr int RPI = 64 / CPR;                   // rows per store instruction
+#pragma unroll
+                for (int i = 0; i < 32 / RPI; ++i) {
+                    const int row = RPI * i + lane_e / CPR, chunk = lane_e % CPR;
+                    const u32x4 w = *(const lds_u32x4 *)(uintptr_t)(obase + row * ROWB + ((chunk ^ (row & (CPR - 1))) << 4));
+                    *reinterpret_cast<u32x4 *>(Oh + (size_t)(qw + row) * o_rs + 8 * chunk) = w;
+                }
+            } else {
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -1143,11 +1179,13 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     *reinterpret_cast<u32x2 *>(Oh + (GENERAL ? (size_t)row_head[b] * a.o_hs + (size_t)row_pos[b] * o_rs : (size_t)q * o_rs) +
                                                32 * db + 8 * g + 4 * half) = w;
                 }
+            }
             if (a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
         }
     }
     FA_TL(5);
-    if (fr1 > fr0)    // the last iteration ended with a barrier: the LDS behind the first LA K stages is free
+    if (!GENERAL && fr1 > fr0) __syncthreads();       // (the epilogue's LDS blocks have been read by their waves)
+    if (fr1 > fr0)    // the LDS behind the first LA K stages is free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      fr0, fr1, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
                                      a.seed_lo, a.seed_hi, (uint32_t)bh, lds0 + LA * TILEB);
