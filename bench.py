@@ -21,8 +21,8 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 
 # HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
-# worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 432.3 MB read + 141.2 MB written.
-MEASURED_HBM_BYTES = {"c3": 574.1e6, "c2": 68.2e6, "c4": 766.7e6}
+# worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 437.5 MB read + 136.4 MB written.
+MEASURED_HBM_BYTES = {"c3": 573.9e6, "c2": 68.2e6, "c4": 780.4e6}
 TRAFFIC_SOURCE = {"c3": "profiles/fa_fwd_pipelined_c3_pmc.md", "c2": "profiles/fa_fwd_pipelined_c2_pmc.md",
                   "c4": "profiles/fa_fwd_pipelined_c4_pmc.md"}
 # the same for the two backward kernels together on c3's shape: 1756.4 MB read + 414.9 MB written
