@@ -319,8 +319,9 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     a.o_part = static_cast<float *>(workspace);
     a.lse_part = a.o_part != nullptr ? a.o_part + (size_t)a.n_splits * p->B * p->N * p->S * p->d : nullptr;
     a.pack = packed_group(p);
-    bool general = a.Hk != p->N || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
-    bool strided = false;       // the regular problem, not stored contiguous [B,N,S,d]
+    bool general = a.pack > 1 || p->S % 128 != 0 || a.Sk != p->S || a.n_splits > 1;
+    // the regular problem, not stored contiguous [B,N,S,d], or with K/V heads shared by groups of query heads
+    bool strided = a.Hk != p->N;
     {
         const long long *strides[4] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides};
         long long eff[4][3];

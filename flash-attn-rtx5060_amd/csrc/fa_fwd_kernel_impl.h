@@ -399,6 +399,24 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 // feeds two matrix instructions, and the wave needs the whole 512-entry
 // register file of its SIMD (one wave per SIMD).
 // ---------------------------------------------------------------------------
+// List head index `bh` (batch * heads + position in the batch entry's list) -> batch entry, query head and K/V
+// head of a strided-layout work item.  With as many K/V heads as query heads the list position is the head;
+// with groups of H / Hk query heads per K/V head, position r stands for K/V head r % Hk and the (r / Hk)-th
+// query head of its group.  (32-bit unsigned divisions; all operands are uniform.)
+__device__ __forceinline__ int fa_strided_heads(int bh, int H, int Hk, int *hi, int *hk)
+{
+    const unsigned bi = (unsigned)bh / (unsigned)H, r = (unsigned)bh - bi * (unsigned)H;
+    unsigned q = r, k = r;
+    if (Hk != H) {
+        const unsigned member = r / (unsigned)Hk;
+        k = r - member * (unsigned)Hk;
+        q = k * ((unsigned)H / (unsigned)Hk) + member;
+    }
+    *hi = (int)q;
+    *hk = (int)k;
+    return (int)bi;
+}
+
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
 template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>
@@ -552,10 +570,14 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         Oh = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs;
     } else {
         if (STRIDED) {
-        const int bi = bh / a.H, hi = bh - bi * a.H;
+        // (grouped K/V heads as in the general kernels: the list walks the K/V heads fastest, so that the query
+        // heads of one K/V head run on the XCD whose L2 holds its K and V)
+        int hi, hk;
+        const int bi = fa_strided_heads(bh, a.H, a.Hk, &hi, &hk);
+        bh = bi * a.H + hi;         // from here on the real head index (logsumexp, ALiBi slope)
         Qh = a.Q + (size_t)bi * a.q_bs + (size_t)hi * a.q_hs;
-        Kh = a.K + (size_t)bi * a.k_bs + (size_t)hi * a.k_hs;
-        Vh = a.V + (size_t)bi * a.v_bs + (size_t)hi * a.v_hs;
+        Kh = a.K + (size_t)bi * a.k_bs + (size_t)hk * a.k_hs;
+        Vh = a.V + (size_t)bi * a.v_bs + (size_t)hk * a.v_hs;
         Oh = a.O + (size_t)bi * a.o_bs + (size_t)hi * a.o_hs;
         } else {
         const size_t head_off = (size_t)bh * S * D;
@@ -1075,10 +1097,11 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         fa_item_decode(next_item, a.BH, a.n_qblocks, a.descending, &nbh, &nqb);
         const uint16_t *nQ, *nK, *nV;
         if (STRIDED) {
-            const int nbi = nbh / a.H, nhi = nbh - nbi * a.H;
+            int nhi, nhk;
+            const int nbi = fa_strided_heads(nbh, a.H, a.Hk, &nhi, &nhk);
             nQ = a.Q + (size_t)nbi * a.q_bs + (size_t)nhi * a.q_hs;
-            nK = a.K + (size_t)nbi * a.k_bs + (size_t)nhi * a.k_hs;
-            nV = a.V + (size_t)nbi * a.v_bs + (size_t)nhi * a.v_hs;
+            nK = a.K + (size_t)nbi * a.k_bs + (size_t)nhk * a.k_hs;
+            nV = a.V + (size_t)nbi * a.v_bs + (size_t)nhk * a.v_hs;
         } else {
             const size_t noff = (size_t)nbh * S * D;
             nQ = a.Q + noff; nK = a.K + noff; nV = a.V + noff;

@@ -24,7 +24,7 @@ struct FaKernelArgs {
     float scale_log2e;   // softmax scale * log2(e)
     long long n_items;   // work items: BH * n_qblocks
     unsigned *queue;     // null, or 9 counters of a work queue: next list position per XCD [0..7], finished workgroups [8]
-    // --- used by the GENERAL instantiations only (strides in elements; the head dimension is contiguous)
+    // --- used by the GENERAL and STRIDED instantiations only (strides in elements; the head dimension is contiguous)
     int Hk;              // K/V heads per batch entry; query head h reads K/V head h / (H / Hk)
     int q_rs, k_rs, v_rs, o_rs;                 // row (sequence position) strides
     long long q_bs, q_hs, k_bs, k_hs;           // batch and head strides

@@ -84,6 +84,35 @@ def test_grouped_query_heads(fa, oracle, H, Hk, S, D, dtype, causal, wl):
         assert torch.equal(o3.view(torch.int16), o4.view(torch.int16))
 
 
+@pytest.mark.parametrize("H,Hk,S,D,dtype,bshd,wl", [(8, 2, 512, 128, 0, False, -1), (16, 8, 768, 64, 1, True, 200),
+                                                       (4, 1, 256, 128, 0, True, -1), (12, 4, 1280, 128, 0, False, 300)])
+def test_grouped_heads_with_alibi_in_the_regular_shape(fa, oracle, H, Hk, S, D, dtype, bshd, wl):
+    """Grouped K/V heads at a length that is a multiple of 128 with S_kv = S take the kernels of the regular
+    problem (strided flavour: the K/V head of a work item comes from its list position).  Slopes differ per query
+    head, so a wrong head index shows; the run with K/V expanded to one head per query head must give the same
+    bits, and so must every schedule."""
+    import torch
+    B = 2
+    q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=900 + H)
+    _, k, v = make_inputs(fa, (B, Hk, S, D), dtype, seed=901 + H)
+    slopes = (np.power(2.0, -8.0 / H * (np.arange(H) + 1)) * np.where(np.arange(H) % 3 == 0, -1.0, 1.0)).astype(np.float32)
+    if bshd:
+        tq, tk, tv = (to_torch(np.ascontiguousarray(x.transpose(0, 2, 1, 3)), dtype).transpose(1, 2) for x in (q, k, v))
+    else:
+        tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    o, lse = run_and_check(fa, oracle, q, k, v, dtype, tq, tk, tv, True, wl, -1, slopes, what=f"GQA {H}/{Hk} ALiBi")
+    rep = H // Hk
+    ts = torch.from_numpy(slopes).cuda()
+    o2, lse2 = fa.flash_attention_forward(to_torch(q, dtype), to_torch(k, dtype).repeat_interleave(rep, dim=1),
+                                          to_torch(v, dtype).repeat_interleave(rep, dim=1), causal=True, window_left=wl, alibi_slopes=ts)
+    torch.cuda.synchronize()
+    assert torch.equal(o.contiguous().view(torch.int16), o2.view(torch.int16)) and torch.equal(lse, lse2)
+    for sched in (1, 2, 3):
+        o3, lse3 = fa.flash_attention_forward(tq, tk, tv, causal=True, window_left=wl, alibi_slopes=ts, sched=sched)
+        torch.cuda.synchronize()
+        assert torch.equal(o.view(torch.int16), o3.view(torch.int16)) and torch.equal(lse, lse3), sched
+
+
 def test_padded_rows_and_everything_at_once(fa, oracle):
     """Row stride larger than the head dimension (a slice of a wider tensor), [B,S,H,D] storage, grouped K/V
     heads, a ragged length, causal + left window and ALiBi in one launch."""
