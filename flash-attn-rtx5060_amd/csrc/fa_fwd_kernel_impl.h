@@ -710,15 +710,17 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
 #pragma unroll
     for (int b = 0; b < RB; ++b) { m_run[b] = -INFINITY; l_a[b] = 0.0f; l_b[b] = 0.0f; }
-    // Without ALiBi the tile scores stay raw dot products and the softmax scale is folded into the exponent
-    // (exp2(s*c - m*c)).  With ALiBi a tile is first rewritten in place to log2 units with the bias applied,
-    // s*c - slope*log2(e)*|i-j| (mask.h:21-26 subtracts slope*|i-j| from the scaled score), so maxima, the
-    // reference point and the exponent work on those values with a factor of one.
+    // The tile scores stay raw dot products and the softmax scale is folded into the exponent (exp2(s*c - m*c)).
+    // ALiBi (mask.h:21-26 subtracts slope*|i-j| from the scaled score) enters through the matrix instruction's
+    // accumulator: the first product of a key block starts from -(slope/scale)*|i-j| instead of from zero, two
+    // vector instructions per score element in front of that instruction, and everything behind it is the code
+    // of the kernels without ALiBi.  (Rewriting the finished tile, s*c - slope*log2(e)*|i-j|, took three per
+    // element in the serial phase of the iteration.)
     const float c = a.scale_log2e;
-    const float cs = ALIBI ? 1.0f : c;
+    const float cs = c;
     // (one slope per head: per lane when the rows of a wave belong to several heads of a packed group)
     const float slope = ALIBI ? a.alibi[bh % a.H + (GENERAL ? row_head[0] : 0)] : 0.0f;
-    const float slope_l2 = slope * 1.44269504088896340736f;
+    const float neg_slope_raw = ALIBI ? -slope / a.scale : 0.0f;        // per key of distance, in raw score units
     const float thresh = kRescaleLog2 / cs;
     uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
     f32x16 sx[RB][2];           // S^T of the tile whose softmax comes next: [key block 0 / 1]
@@ -748,18 +750,22 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             }
         }
     };
-    auto apply_alibi = [&](int tile) __attribute__((always_inline)) {
+    // the initial accumulator of key block `blk` of `tile` for row block b
+    auto alibi_start = [&](int b, int blk, int tile) __attribute__((always_inline)) {
+        // signed distance of this lane's query to the lane's first key of the block: exact in fp32
+        const float base = (float)(row_pos[b] + pos_off - (tile * kBlockKeys + 32 * blk + 4 * half));
+        f32x16 v;
+        if (MASKED && a.R == 0) {
+            // no visible key lies behind its query: the distance is base - k without the absolute value (the
+            // elements for which that is wrong are masked), one fused multiply-add with the key offset as a literal
+            const float at_base = base * neg_slope_raw;
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            // signed distance of this lane's query to the lane's first key of the tile: exact in fp32
-            const float base = (float)(row_pos[b] + pos_off - (tile * kBlockKeys + 4 * half));
+            for (int r = 0; r < 16; ++r) v[r] = __builtin_fmaf((float)(8 * (r >> 2) + (r & 3)), -neg_slope_raw, at_base);
+        } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float k0 = (float)(8 * (r >> 2) + (r & 3));
-                sx[b][0][r] = __builtin_fmaf(__builtin_fabsf(base - k0), -slope_l2, sx[b][0][r] * c);
-                sx[b][1][r] = __builtin_fmaf(__builtin_fabsf(base - (k0 + 32.0f)), -slope_l2, sx[b][1][r] * c);
-            }
+            for (int r = 0; r < 16; ++r) v[r] = __builtin_fabsf(base - (float)(8 * (r >> 2) + (r & 3))) * neg_slope_raw;
         }
+        return v;
     };
     auto row_max = [&](int b) __attribute__((always_inline)) {
         float mx = fmaxf(sx[b][0][0], sx[b][1][0]);
@@ -829,7 +835,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
         if (RB == 2) mfma_result_wait();       // the epilogue may follow
     };
-    auto qk_plain = [&](int kstage) __attribute__((always_inline)) {
+    auto qk_plain = [&](int kstage, int tile) __attribute__((always_inline)) {
         const uint32_t ks = kstage * TILEB;
         u32x4 fr[NQK];
         fr[0] = read_k(ks, 0);
@@ -838,6 +844,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int b = 0; b < RB; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) { sx[b][0][r] = 0.0f; sx[b][1][r] = 0.0f; }
+        if (ALIBI) {
+#pragma unroll
+            for (int b = 0; b < RB; ++b) { sx[b][0] = alibi_start(b, 0, tile); sx[b][1] = alibi_start(b, 1, tile); }
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < NQK; ++n) {
@@ -869,7 +879,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
         if (DROPOUT) draw_dropout(tile);
-        if (ALIBI) apply_alibi(tile);
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
@@ -903,7 +912,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int n = 0; n < PD; ++n) fetch(n);
         if (DROPOUT) draw_dropout(tile);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
-        if (ALIBI) apply_alibi(tile);
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
         bool moved[RB];
         float alpha[RB], nmc[RB];
@@ -929,7 +937,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                     if (RB == 2 && n < 2) PinnedMfma<BF16>::qk_first(nx[b][n & 1], fr[g], qf[b][n >> 1]);
                     else if (RB == 2) PinnedMfma<BF16>::qk_next(nx[b][n & 1], fr[g], qf[b][n >> 1]);
-                    else nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n < 2 ? zero : nx[b][n & 1]);
+                    else nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n >= 2 ? nx[b][n & 1] : ALIBI ? alibi_start(b, n & 1, tile + 1) : zero);
                 }
                 // softmax work riding along: the 16*RB element pairs of this tile spread over the NF*RB matrix
                 // instructions, row block 0 first (its registers are free again when S^T(tile+1) is born)
@@ -946,8 +954,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
                     const float x0 = e < 8 ? sx[pb][0][2 * e] : sx[pb][1][2 * (e - 8)];
                     const float x1 = e < 8 ? sx[pb][0][2 * e + 1] : sx[pb][1][2 * (e - 8) + 1];
                     asm volatile("" : "+v"(nmc[pb]));
-                    const float e0 = __builtin_amdgcn_exp2f(ALIBI ? x0 + nmc[pb] : __builtin_fmaf(x0, c, nmc[pb]));
-                    const float e1 = __builtin_amdgcn_exp2f(ALIBI ? x1 + nmc[pb] : __builtin_fmaf(x1, c, nmc[pb]));
+                    const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, nmc[pb]));
+                    const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, nmc[pb]));
                     l_a[pb] += e0;
                     l_b[pb] += e1;
                     uint32_t packed = N::pack2(dropped(e0, pb, e >> 3, 2 * (e & 7)), dropped(e1, pb, e >> 3, 2 * (e & 7) + 1));
@@ -1022,7 +1030,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (more_v) issue_v(tv, jm3);              // (j - 2 + LA) % NST == (j - 3) % NST
         if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(jm2);
         if (my_lo <= i && i <= my_hi) softmax_plain(i);
-        if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3);
+        if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3, i + 1);
         finish_iteration(more_k && more_v, tv > t1);
     };
     auto steady_iteration = [&](auto J3, int i) __attribute__((always_inline)) {
@@ -1144,7 +1152,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
             const float inv = empty ? 0.0f : 1.0f / l_tot;
             const float lse_row = empty ? -INFINITY
-                                        : m_run[b] * (ALIBI ? 0.69314718055994530942f : a.scale) + __builtin_logf(l_tot);
+                                        : m_run[b] * a.scale + __builtin_logf(l_tot);
             if (GENERAL && o_part != nullptr) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
