@@ -62,6 +62,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBlockKeys = 64;          // keys per K/V tile
+constexpr float kNoReference = -1.0e30f; // reference point of a row before its first visible score
 constexpr float kRescaleLog2 = 8.0f;    // rescale O only when a row max grew by > 2^8
 
 template <bool BF16> struct Num;
@@ -126,6 +127,24 @@ template <int CPR> __device__ __forceinline__ int k_swz(int row) { return CPR ==
 // consecutive chunks; the 4 rows must land on 4 different 64-byte bank groups.
 template <int CPR> __device__ __forceinline__ int v_swz(int row) { return CPR == 16 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 
+// max(x of lane l, x of lane l^32), in both lanes: after v_permlane32_swap of two copies one register holds the
+// lower half's values in both halves and the other the upper half's.  (The maximum as an instruction of its own:
+// written as fmaxf the compiler first quiets possible signalling NaNs in both operands, an instruction each.)
+__device__ __forceinline__ float max_plain(float a, float b)
+{
+    float m;
+    asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(a), "v"(b));
+    return m;
+}
+// (One assembly statement: handed the two results of __builtin_amdgcn_permlane32_swap, an inline-assembly
+// v_max_f32 received the first of them twice (hipcc 7.2).  The s_nop covers the wait states the swap needs
+// behind the vector instructions that wrote its operands.)
+__device__ __forceinline__ float max_of_halves(float x)
+{
+    float a = x, b = x, m;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_max_f32 %2, %0, %1" : "+v"(a), "+v"(b), "=v"(m));
+    return m;
+}
 __device__ __forceinline__ float swap_halves(float x)
 {
     // lane l <-> lane l^32
@@ -709,7 +728,9 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             for (int r = 0; r < 16; ++r) o[b][db][r] = 0.0f;
     float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
 #pragma unroll
-    for (int b = 0; b < RB; ++b) { m_run[b] = -INFINITY; l_a[b] = 0.0f; l_b[b] = 0.0f; }
+    // (the reference point starts from a finite value far below every score: the first finite row maximum moves
+    // it, with a factor exp2(-huge) = 0 for the empty accumulators, and no place needs a test for -inf)
+    for (int b = 0; b < RB; ++b) { m_run[b] = kNoReference; l_a[b] = 0.0f; l_b[b] = 0.0f; }
     // The tile scores stay raw dot products and the softmax scale is folded into the exponent (exp2(s*c - m*c)).
     // ALiBi (mask.h:21-26 subtracts slope*|i-j| from the scaled score) enters through the matrix instruction's
     // accumulator: the first product of a key block starts from -(slope/scale)*|i-j| instead of from zero, two
@@ -768,20 +789,20 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         return v;
     };
     auto row_max = [&](int b) __attribute__((always_inline)) {
-        float mx = fmaxf(sx[b][0][0], sx[b][1][0]);
+        float mx = max_plain(sx[b][0][0], sx[b][1][0]);
 #pragma unroll
         for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, sx[b][0][r]), sx[b][1][r]);
-        return fmaxf(mx, swap_halves(mx));
+        return max_of_halves(mx);
     };
     // the decision to move the reference point of row block b; returns the factor by which everything
     // accumulated so far has to be multiplied (1 when the reference point stays)
     auto new_reference = [&](int b, float mx, bool &moved) __attribute__((always_inline)) {
         float alpha = 1.0f;
-        const bool grow = mx > m_run[b] + thresh;   // -inf + thresh = -inf: a first finite max always grows
+        const bool grow = mx > m_run[b] + thresh;   // (from kNoReference every finite maximum grows)
         moved = __builtin_amdgcn_ballot_w64(grow) != 0;
         if (moved) {
             const float m_new = grow ? mx : m_run[b];
-            alpha = (m_run[b] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run[b] - m_new) * cs);
+            alpha = __builtin_amdgcn_exp2f((m_run[b] - m_new) * cs);
             l_a[b] *= alpha;
             l_b[b] *= alpha;
             m_run[b] = m_new;
@@ -885,7 +906,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
             bool moved;
             const float alpha = new_reference(b, row_max(b), moved);
             if (moved) scale_o(b, alpha);
-            const float mc = (m_run[b] == -INFINITY) ? 0.0f : m_run[b] * cs;
+            const float mc = m_run[b] * cs;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], cs, -mc));
@@ -918,7 +939,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
         for (int b = 0; b < RB; ++b) {
             alpha[b] = new_reference(b, row_max(b), moved[b]);
-            nmc[b] = (m_run[b] == -INFINITY) ? 0.0f : -m_run[b] * cs;
+            nmc[b] = -m_run[b] * cs;
         }
         uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
         f32x16 nx[RB][2];                          // S^T(tile+1)
