@@ -48,7 +48,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd_validate", "fa_fwd", "fa_init", "fa_fwd_split_static", "fa_fwd_static_scratch_bytes",
     "fa_reset_work_queues", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
-    "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
+    "fa_sched_heads", "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
     "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_algorithmic_flops",
     "fa_bwd_sched_query_tile_range", "fa_bwd_sched_classify",
@@ -141,6 +141,7 @@ def lib():
         L.fa_sched_num_items.argtypes = [ctypes.c_int] * 4
         L.fa_sched_item.argtypes = [ctypes.c_int] * 7 + [ctypes.c_longlong, ctypes.POINTER(ctypes.c_int),
                                                          ctypes.POINTER(ctypes.c_int)]
+        L.fa_sched_heads.argtypes = [ctypes.c_int] * 3 + [ctypes.POINTER(ctypes.c_int)] * 3
         L.fa_sched_tile_range.restype = None
         L.fa_sched_tile_range.argtypes = [ctypes.c_int] * 7 + [ctypes.POINTER(ctypes.c_int)] * 2
         L.fa_sched_classify.argtypes = [ctypes.c_int] * 7

@@ -135,6 +135,14 @@ int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left, in
     return FA_OK;
 }
 
+int fa_sched_heads(int N, int n_kv_heads, int bh, int *batch, int *q_head, int *kv_head)
+{
+    const int hk = n_kv_heads > 0 ? n_kv_heads : N;
+    if (N <= 0 || hk > N || N % hk != 0 || bh < 0 || !batch || !q_head || !kv_head) return FA_ERR_BAD_SHAPE;
+    *batch = fa_strided_heads(bh, N, hk, q_head, kv_head);
+    return FA_OK;
+}
+
 void fa_sched_tile_range(int S, int block_keys, int is_causal, int window_left, int window_right,
                          int q_begin, int rows, int *tile_lo, int *tile_hi)
 {

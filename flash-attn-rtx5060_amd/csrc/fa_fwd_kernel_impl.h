@@ -418,24 +418,6 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 // feeds two matrix instructions, and the wave needs the whole 512-entry
 // register file of its SIMD (one wave per SIMD).
 // ---------------------------------------------------------------------------
-// List head index `bh` (batch * heads + position in the batch entry's list) -> batch entry, query head and K/V
-// head of a strided-layout work item.  With as many K/V heads as query heads the list position is the head;
-// with groups of H / Hk query heads per K/V head, position r stands for K/V head r % Hk and the (r / Hk)-th
-// query head of its group.  (32-bit unsigned divisions; all operands are uniform.)
-__device__ __forceinline__ int fa_strided_heads(int bh, int H, int Hk, int *hi, int *hk)
-{
-    const unsigned bi = (unsigned)bh / (unsigned)H, r = (unsigned)bh - bi * (unsigned)H;
-    unsigned q = r, k = r;
-    if (Hk != H) {
-        const unsigned member = r / (unsigned)Hk;
-        k = r - member * (unsigned)Hk;
-        q = k * ((unsigned)H / (unsigned)Hk) + member;
-    }
-    *hi = (int)q;
-    *hk = (int)k;
-    return (int)bi;
-}
-
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
 template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>

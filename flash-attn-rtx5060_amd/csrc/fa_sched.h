@@ -82,4 +82,24 @@ FA_HD void fa_item_decode(long long item, int BH, int n_qblocks, int descending,
     *qblock = descending ? (n_qblocks - 1 - (int)rank) : (int)rank;
 }
 
+// List head index `bh` (batch * heads + position in the batch entry's list) -> batch entry, query head and K/V
+// head of a work item of the regular problem with grouped K/V heads.  With as many K/V heads as query heads the
+// list position is the head; with groups of H / Hk query heads per K/V head, position r stands for K/V head
+// r % Hk and the (r / Hk)-th query head of its group: the list walks the K/V heads fastest, so that with the
+// head index dealt round robin over the XCDs (fa_item_decode) the query heads of one K/V head run on the XCD
+// whose L2 holds its K and V.  (32-bit unsigned divisions; all operands are uniform.)
+FA_HD int fa_strided_heads(int bh, int H, int Hk, int *hi, int *hk)
+{
+    const unsigned bi = (unsigned)bh / (unsigned)H, r = (unsigned)bh - bi * (unsigned)H;
+    unsigned q = r, k = r;
+    if (Hk != H) {
+        const unsigned member = r / (unsigned)Hk;
+        k = r - member * (unsigned)Hk;
+        q = k * ((unsigned)H / (unsigned)Hk) + member;
+    }
+    *hi = (int)q;
+    *hk = (int)k;
+    return (int)bi;
+}
+
 #endif

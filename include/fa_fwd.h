@@ -215,6 +215,12 @@ long long fa_sched_num_items(int B, int N, int S, int d);
 /* Work item `item` (0 = launched first) -> batch*N+head and first query row. */
 int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left,
                   int window_right, long long item, int *bh, int *q_begin);
+/* Grouped K/V heads of the regular problem (S a multiple of 128, S_kv = S, no key splits): the `bh` that
+ * fa_sched_item returns is a position in the list of heads, and the kernel turns it into batch entry, query head
+ * and K/V head like this (K/V heads fastest, so that the query heads of a K/V head share an XCD's L2).  With
+ * n_kv_heads = 0 or N the position is the head.  No counterpart in the reference, which has one K/V head per
+ * query head (flash_forward.h:378-381). */
+int fa_sched_heads(int N, int n_kv_heads, int bh, int *batch, int *q_head, int *kv_head);
 /* Key-tile range [*tile_lo, *tile_hi] (inclusive) visited for query rows
  * [q_begin, q_begin + rows).  Same clipping as flash_forward.h:52-61. */
 void fa_sched_tile_range(int S, int block_keys, int is_causal, int window_left,

@@ -114,3 +114,22 @@ def test_pair_counts_and_flops(fa):
     assert L.fa_count_pairs(16384, 1, 1024, -1) == 16268800
     assert L.fa_count_pairs(32768, 1, -1, -1) == 536887296
     assert abs(L.fa_algorithmic_flops(2, 32, 8192, 128, 1, -1, -1) - 1.0996e12) < 1e8
+
+
+@pytest.mark.parametrize("N,Nk", [(8, 8), (8, 2), (8, 1), (32, 8), (12, 4), (6, 3), (5, 0)])
+def test_grouped_heads_list_walks_the_kv_heads_fastest(fa, N, Nk):
+    """Every (batch entry, query head) once; query head h reads K/V head h / (N / Nk) (include/fa_fwd.h,
+    n_kv_heads); consecutive list positions inside a group of Nk belong to consecutive K/V heads."""
+    L = fa.lib()
+    hk = Nk if Nk > 0 else N
+    group = N // hk
+    seen = set()
+    b, q, k = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    for bh in range(3 * N):
+        assert L.fa_sched_heads(N, Nk, bh, ctypes.byref(b), ctypes.byref(q), ctypes.byref(k)) == 0
+        assert b.value == bh // N and 0 <= q.value < N and k.value == q.value // group
+        assert k.value == (bh % N) % hk
+        seen.add((b.value, q.value))
+    assert len(seen) == 3 * N
+    assert L.fa_sched_heads(8, 3, 0, ctypes.byref(b), ctypes.byref(q), ctypes.byref(k)) != 0      # 3 does not divide 8
+    assert L.fa_sched_heads(8, 2, -1, ctypes.byref(b), ctypes.byref(q), ctypes.byref(k)) != 0
