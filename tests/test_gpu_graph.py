@@ -42,6 +42,38 @@ def test_forward_and_backward_replayed_from_a_graph(fa, shape, sched):
                                b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)), (replay, shape, sched)
 
 
+@pytest.mark.parametrize("sched", [0, 3])
+def test_grouped_heads_in_bshd_storage_with_alibi_replayed_from_a_graph(fa, sched):
+    """The strided flavour of the regular kernels (tensors stored [B,S,H,D], 8 query heads on 2 K/V heads, ALiBi
+    slopes) captured once and replayed on new contents: every replay equals an eager call bit for bit."""
+    import numpy as np
+    import torch
+    B, H, Hk, S, D = 2, 8, 2, 1024, 128
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q = torch.randn((B, S, H, D), device="cuda", generator=g).half().transpose(1, 2)
+    k, v = (torch.randn((B, S, Hk, D), device="cuda", generator=g).half().transpose(1, 2) for _ in range(2))
+    slopes = torch.from_numpy(np.power(2.0, -8.0 / H * (np.arange(H) + 1)).astype(np.float32)).cuda()
+    o = torch.empty((B, S, H, D), device="cuda", dtype=torch.float16).transpose(1, 2)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+    kw = dict(causal=True, window_left=300, alibi_slopes=slopes, sched=sched)
+    fa.flash_attention_forward(q, k, v, out=o, lse=lse, **kw)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            fa.flash_attention_forward(q, k, v, out=o, lse=lse, **kw)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for t in (q, k, v):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=g).half())
+        graph.replay()
+        torch.cuda.synchronize()
+        o2, lse2 = fa.flash_attention_forward(q, k, v, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(o.contiguous().view(torch.int16), o2.contiguous().view(torch.int16)) and torch.equal(lse, lse2), (replay, sched)
+
+
 def test_more_captured_queue_launches_than_counter_sets(fa):
     """Every captured queue launch owns a counter set; a device has 240 of them for captured launches, further ones
     walk the fixed order.  300 launches captured into one graph, replayed three times on new inputs: every launch's
