@@ -267,6 +267,24 @@ template <bool BF16> __device__ __forceinline__ f32x2 storage_product2(uint32_t 
     return f32x2{__builtin_bit_cast(float, r << 16), __builtin_bit_cast(float, r & 0xffff0000u)};
 }
 
+// s0 += a.lo * b.lo and s1 += a.hi * b.hi with every product rounded to the storage type first (s0 and s1 may be
+// the same sum: the low product is then added before the high one).  fp16: the rounded pair from v_pk_mul_f16 goes
+// into the fp32 sums through v_fma_mix_f32 (x * 1.0 + sum with the half-precision operand widened on the way:
+// the same bits as a conversion followed by an addition, in one instruction instead of two).
+template <bool BF16> __device__ __forceinline__ void add_storage_products(uint32_t a, uint32_t b, float &s0, float &s1)
+{
+    if (!BF16) {
+        f16x2 pr = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
+        uint32_t bits = __builtin_bit_cast(uint32_t, pr);
+        asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "+v"(s0) : "v"(bits));
+        asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(s1) : "v"(bits));
+        return;
+    }
+    const f32x2 pr = storage_product2<BF16>(a, b);
+    s0 += pr[0];
+    s1 += pr[1];
+}
+
 // Queries row0..row1-1 of a head (query i at key position i + pos_off, all positions below 32) against keys
 // 0..31.  The 32 x D blocks of Q, K and V (the rows needed) are staged in LDS once (K with its 16-byte chunks
 // XOR-swizzled by the row, so that 32 lanes reading one chunk of 32 different rows do not collide), everything
@@ -322,9 +340,7 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        const f32x2 pr = storage_product2<BF16>(qa[c][w], kb[c][w]);
-                        sum += pr[0];
-                        sum += pr[1];
+                        add_storage_products<BF16>(qa[c][w], kb[c][w], sum, sum);
                     }
             }
             s = sum * scale;
@@ -394,9 +410,7 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 #pragma unroll
         for (int j = 0; j < R; ++j) {
             if (j >= lo && j <= p) {
-                const f32x2 pr = storage_product2<BF16>(pw[j], vw[j]);
-                s0 += pr[0];
-                s1 += pr[1];
+                add_storage_products<BF16>(pw[j], vw[j], s0, s1);
             }
         }
         const uint32_t packed = Num<BF16>::pack2(s0, s1);
