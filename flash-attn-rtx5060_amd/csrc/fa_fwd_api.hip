@@ -368,16 +368,21 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     a.queue = nullptr;
     const long long resident = (long long)ds->compute_units * (waves == 8 ? 1 : 2);
     // FA_SCHED_AUTO: with at most one item per resident workgroup there is nothing to schedule (and the
-    // queue's counter round trips, 2.3 us each, would double the run time of a 7 us problem); with at most
-    // two, the fixed snake pairs every long item with a short one; beyond that the work queue balances best.
-    // Measured: c1 9.5 / 9.5 / 5.8 TFLOP/s (dispatch / snake / queue), c2 431 / 611 / 448, c3 995 / 955 / 1030.
+    // queue's counter round trips, 2.3 us each, would double the run time of a 7 us problem).  With fewer than
+    // eight items per workgroup the fixed snake wins: it pairs every long item with a short one, knows its next
+    // item without asking, and its items' loads can be requested before the current item's epilogue without a
+    // counter in between -- causal fp16 problems, snake against queue: B8 H32 S1024 D64 (four items per workgroup)
+    // 67 against 100 us, B4 H32 S2048 D64 (four) 111 against 138, B2 H32 S4096 D128 (four) 290 against 312, c2 (two)
+    // 611 against 448 TFLOP/s.  At eight per workgroup the two are level (c3 1016 against 1018 TFLOP/s, B1 H32 S16384
+    // 2097 us both); beyond, the queue's balancing is worth more than its counters cost (c5, 32 items per workgroup:
+    // 16.2 against 17.0 ms; B8 H32 S8192 D64 2.75 against 2.80 ms).
     int sched = p->sched;
     // Items that are all alike (no mask, or a window of at most half the length: all but the first few query blocks
     // of a head see the same number of tiles) need no balancing either, and the fixed order saves them the
     // counters' barriers: c4 766 against 748 TFLOP/s, c3's shape without a mask 1101 against 1096.
     if (sched == FA_SCHED_AUTO) {
         const bool alike = !a.descending || 2LL * a.L <= (long long)p->S;
-        sched = a.n_items <= resident ? FA_SCHED_DISPATCH : (a.n_items <= 2 * resident || alike) ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
+        sched = a.n_items <= resident ? FA_SCHED_DISPATCH : (a.n_items < 8 * resident || alike) ? FA_SCHED_PERSISTENT : FA_SCHED_QUEUE;
     }
     if (sched == FA_SCHED_PERSISTENT || sched == FA_SCHED_QUEUE) {
         if (grid > resident) grid = resident;

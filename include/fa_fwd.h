@@ -47,7 +47,8 @@ enum { FA_DTYPE_F16 = 0, FA_DTYPE_BF16 = 1 };
 /* How work items (batch, head, query block) reach the compute units. */
 enum {
     FA_SCHED_AUTO = 0,        /* the library picks by the number of work items per resident
-                                 workgroup: <= 1 dispatch, <= 2 persistent, else queue         */
+                                 workgroup: <= 1 dispatch, < 8 (or items all alike) persistent,
+                                 else queue                                                    */
     FA_SCHED_DISPATCH = 1,    /* one workgroup per work item, launched longest-first          */
     FA_SCHED_PERSISTENT = 2,  /* a resident grid sized to the CUs walks the longest-first list
                                  in a fixed snake order                                       */
