@@ -29,8 +29,9 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
-hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, hipStream_t stream);
-hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, hipStream_t stream);
+hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, int compute_units,
+                              hipStream_t stream);
+hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream);
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -571,8 +572,8 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
 {
     const int st = fa_bwd_validate(p);
     if (st != FA_OK) return st;
+    const FaDeviceState *ds = nullptr;
     {
-        const FaDeviceState *ds = nullptr;
         const hipError_t de = fa_device_state(&ds);
         if (de != hipSuccess) return device_fail(de, "device set-up");
     }
@@ -623,9 +624,10 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.seed_hi = (unsigned)(p->seed >> 32);
     const int masked = (general || a.L < far || a.R < far) ? 1 : 0;
     hipError_t e = a.drop_threshold != 0
-        ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, static_cast<hipStream_t>(stream))
+        ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, ds->compute_units,
+                                     static_cast<hipStream_t>(stream))
         : fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general ? 1 : 0, a.alibi != nullptr ? 1 : 0,
-                             static_cast<hipStream_t>(stream));
+                             ds->compute_units, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
 }
 
