@@ -162,14 +162,14 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     // Work items: one workgroup per item, or (grid smaller than the list) a resident grid that walks the
     // longest-first list as a snake, pass 0 forwards, pass 1 backwards, ..., which pairs long items with short ones.
     const long long n_items = (long long)a.B * a.H * n_qblocks;
-    for (int pass = 0;; ++pass) {
+    for (int pass = 0; !GENERAL || pass < 1; ++pass) {      // (general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();          // (the LDS stages: other waves may still be reading the last tile)
     // (the lane index is taken from the hardware once per work item and tied to this place: what is derived from
     // it would otherwise be computed in front of the item loop and kept in registers through every tile loop)
-    int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    asm volatile("" : "+v"(lane));
+    int lane = GENERAL ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (!GENERAL) asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31;
     int bh, qblock;
     fa_item_decode(item, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
@@ -359,12 +359,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // (work items as in fa_bwd_dq; the list here is ascending in the key block, which is longest first under a
     // causal mask: key block 0 is seen by every query)
     const long long n_items = (long long)a.B * a.Hk * n_kblocks;
-    for (int pass = 0;; ++pass) {
+    for (int pass = 0; !GENERAL || pass < 1; ++pass) {      // (general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();
-    int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    asm volatile("" : "+v"(lane));
+    int lane = GENERAL ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (!GENERAL) asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31;
     int bhk, kblock;
     fa_item_decode(item, a.B * a.Hk, n_kblocks, 0, &bhk, &kblock);
@@ -611,7 +611,12 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream)
     // (a window of at most half the length leaves the items alike too: c4's shape 1.14 ms in the hardware's order,
     // 1.16 as a snake)
     const unsigned resident = (unsigned)compute_units;
-    const bool uneven = MASKED && 2LL * a.L > (long long)a.S;
+    // (the general instantiations always carry the mask code: without a bound on either side, L = R = S + S_kv, their
+    // items are alike as well)
+    const long long unbounded = (long long)a.S + a.Sk;
+    // (The general instantiations are launched one workgroup per item only: with the item loop around them their
+    // 128-wide kernels spill ten times as much and run 15-20 % slower, c3's shape stored [B,S,H,D] 4.7 against 4.0 ms.)
+    const bool uneven = !GENERAL && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
     const unsigned launch_q = (uneven && grid_q > resident && grid_q < 16u * resident) ? resident : grid_q;
     const unsigned launch_k = (uneven && grid_k > resident && grid_k < 16u * resident) ? resident : grid_k;
     hipLaunchKernelGGL(kq, dim3(launch_q), dim3(kBwdWaves * 64), smem_dq, stream, a);
