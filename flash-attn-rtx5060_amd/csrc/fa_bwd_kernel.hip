@@ -1,13 +1,14 @@
 // Backward kernels without dropout: the instantiations for the reference's layout and the general ones.
 #include "fa_bwd_kernel_impl.h"
 
-// general: strides, any lengths, grouped K/V heads (always with the mask code); alibi needs general
+// layout 0: the reference's; 2 (general): strides, any lengths, grouped K/V heads (always with the mask code);
+// alibi needs general.  (Layout 1, strided, is instantiated in a translation unit of its own.)
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, int compute_units,
                               hipStream_t stream)
 {
 #define FA_BWD_CASE(BF, DD, MK, GN, AL) \
     if (bf16 == BF && D == DD && masked == MK && general == GN && alibi == AL) \
-        return launch_bwd<BF != 0, DD, MK != 0, GN != 0, AL != 0, false>(a, compute_units, stream);
+        return launch_bwd<BF != 0, DD, MK != 0, GN != 0 ? 2 : 0, AL != 0, false>(a, compute_units, stream);
     FA_BWD_CASE(0, 64, 0, 0, 0) FA_BWD_CASE(0, 64, 1, 0, 0) FA_BWD_CASE(0, 128, 0, 0, 0) FA_BWD_CASE(0, 128, 1, 0, 0)
     FA_BWD_CASE(1, 64, 0, 0, 0) FA_BWD_CASE(1, 64, 1, 0, 0) FA_BWD_CASE(1, 128, 0, 0, 0) FA_BWD_CASE(1, 128, 1, 0, 0)
     FA_BWD_CASE(0, 64, 1, 1, 0) FA_BWD_CASE(0, 128, 1, 1, 0) FA_BWD_CASE(1, 64, 1, 1, 0) FA_BWD_CASE(1, 128, 1, 1, 0)

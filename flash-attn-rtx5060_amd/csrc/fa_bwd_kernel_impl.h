@@ -12,10 +12,11 @@
 // rescaled logsumexp for the second kernel) and fa_bwd_dkdv (a workgroup owns 256 keys of one K/V head and walks
 // the query tiles of the query heads that share it); no atomics, every output element has one writer, results
 // are the same bits from run to run.
-// Template flags: GENERAL = strides, any lengths (query i at key position i + Sk - S), grouped K/V heads;
-// the other instantiations assume contiguous [B,H,S,D] with S a multiple of 128 and keep their instruction
-// stream free of all that.  ALIBI (GENERAL only) subtracts slope[h] * |position - key| from the scaled score.
-// DROPOUT (GENERAL only) replays the forward pass's keep decisions from (seed, head, query position, key).
+// Template flags: LAYOUT 0 = contiguous [B,H,S,D] with S a multiple of 128 and as many keys; 1 (strided) = the
+// same lengths with row, head and batch strides from the arguments and grouped K/V heads; 2 (general) = that
+// plus any lengths (query i at key position i + Sk - S, ragged last tiles).  Each keeps its instruction stream
+// free of what it does not need.  ALIBI (general only) subtracts slope[h] * |position - key| from the scaled
+// score.  DROPOUT (general only) replays the forward pass's keep decisions from (seed, head, query position, key).
 // Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the
 // lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B operands loaded once into
 // registers, the walked tiles are A operands streamed through LDS by direct global->LDS loads, and an
@@ -130,6 +131,17 @@ __device__ __forceinline__ f32x16 zero16()
     return z;
 }
 
+// The kernel's arguments, read again from the kernel-argument segment: what is taken from the by-value argument
+// is loaded once in front of the item loop and then kept in scalar registers through every tile loop; a use behind
+// this call loads it where it is needed (scalar loads from a segment that stays in the scalar cache).
+__device__ __forceinline__ const FaBwdArgs &args_reloaded()
+{
+    typedef const __attribute__((address_space(4))) FaBwdArgs *KernargPtr;
+    KernargPtr ka = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ka));
+    return *(const FaBwdArgs *)ka;
+}
+
 __device__ __forceinline__ const uint16_t *head_ptr(const uint16_t *p, const FaBwdTensor &t, int b, int h)
 {
     return p + (long long)b * t.bs + (long long)h * t.hs;
@@ -143,9 +155,11 @@ __device__ __forceinline__ uint16_t *head_ptr(uint16_t *p, const FaBwdTensor &t,
 // dQ: a workgroup owns 256 queries (lane = query), walks the key tiles of its visible range.
 // LDS stage: K (read row-wise for S^T = K Q^T and transposed for dQ^T += K^T dS^T), V (row-wise, dP^T = V dO^T).
 // ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI, bool DROPOUT>
+template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a)
 {
+    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
+    static_assert(LAYOUT >= 0 && LAYOUT <= 2, "0 the reference's layout, 1 strided, 2 general");
     static_assert(!GENERAL || MASKED, "the general instantiations always carry the mask code (ragged tiles need it)");
     static_assert(!ALIBI || GENERAL, "ALiBi is instantiated for the general layout only");
     static_assert(!DROPOUT || GENERAL, "dropout is instantiated for the general layout only");
@@ -162,23 +176,23 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     // Work items: one workgroup per item, or (grid smaller than the list) a resident grid that walks the
     // longest-first list as a snake, pass 0 forwards, pass 1 backwards, ..., which pairs long items with short ones.
     const long long n_items = (long long)a.B * a.H * n_qblocks;
-    for (int pass = 0; !GENERAL || pass < 1; ++pass) {      // (general instantiations: exactly one item, no loop)
+    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (strided and general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();          // (the LDS stages: other waves may still be reading the last tile)
     // (the lane index is taken from the hardware once per work item and tied to this place: what is derived from
     // it would otherwise be computed in front of the item loop and kept in registers through every tile loop)
-    int lane = GENERAL ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    if (!GENERAL) asm volatile("" : "+v"(lane));
+    int lane = ONE_ITEM ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (!ONE_ITEM) asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31;
     int bh, qblock;
     fa_item_decode(item, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
-    const int b = bh / a.H, h = bh - b * a.H, hk = GENERAL ? h / (a.H / a.Hk) : h;
-    const int q_rs = GENERAL ? a.q.rs : D, k_rs = GENERAL ? a.k.rs : D, v_rs = GENERAL ? a.v.rs : D;
-    const int o_rs = GENERAL ? a.o.rs : D, g_rs = GENERAL ? a.dO_.rs : D, dq_rs = GENERAL ? a.dq.rs : D;
+    const int b = bh / a.H, h = bh - b * a.H, hk = STRIDES ? h / (a.H / a.Hk) : h;
+    const int q_rs = STRIDES ? a.q.rs : D, k_rs = STRIDES ? a.k.rs : D, v_rs = STRIDES ? a.v.rs : D;
+    const int o_rs = STRIDES ? a.o.rs : D, g_rs = STRIDES ? a.dO_.rs : D, dq_rs = STRIDES ? a.dq.rs : D;
     const uint16_t *Qh, *Kh, *Vh, *Oh, *dOh;
     uint16_t *dQh;
-    if (GENERAL) {
+    if (STRIDES) {
         Qh = head_ptr(a.Q, a.q, b, h); Kh = head_ptr(a.K, a.k, b, hk); Vh = head_ptr(a.V, a.v, b, hk);
         Oh = head_ptr(a.O, a.o, b, h); dOh = head_ptr(a.dO, a.dO_, b, h); dQh = head_ptr(a.dQ, a.dq, b, h);
     } else {
@@ -232,7 +246,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     Reader rd; rd.init(lane, lds0);
     Loader ldk, ldv;
     ldk.init(wave, lane, k_rs * 2);
-    if (GENERAL) ldv.init(wave, lane, v_rs * 2);
+    if (STRIDES) ldv.init(wave, lane, v_rs * 2);
     auto issue = [&](int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
         if (GENERAL && (tile + 1) * 64 > Sk) {
@@ -240,7 +254,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
             ldv.load_ragged(Vh + (size_t)tile * 64 * v_rs, base + TILEB, Sk - tile * 64, v_rs * 2);
         } else {
             ldk.load(Kh + (size_t)tile * 64 * k_rs, base);
-            (GENERAL ? ldv : ldk).load(Vh + (size_t)tile * 64 * v_rs, base + TILEB);
+            (STRIDES ? ldv : ldk).load(Vh + (size_t)tile * 64 * v_rs, base + TILEB);
         }
     };
 
@@ -342,9 +356,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
 // LDS stage: Q (row-wise for S = Q K^T, transposed for dK^T += Q^T dS), dO (row-wise for dP = dO V^T, transposed
 // for dV^T += dO^T P), 64 rescaled logsumexps, 64 deltas.
 // ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI, bool DROPOUT>
+template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
+    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
@@ -353,32 +368,29 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int S = a.S, Sk = GENERAL ? a.Sk : a.S, off = GENERAL ? a.Sk - a.S : 0;
-    const int G = GENERAL ? a.H / a.Hk : 1;
+    const int G = STRIDES ? a.H / a.Hk : 1;
     const int n_kblocks = (Sk + 255) / 256;
     // one K/V head per XCD at a time; key block 0 is seen by the most queries and goes first
     // (work items as in fa_bwd_dq; the list here is ascending in the key block, which is longest first under a
     // causal mask: key block 0 is seen by every query)
     const long long n_items = (long long)a.B * a.Hk * n_kblocks;
-    for (int pass = 0; !GENERAL || pass < 1; ++pass) {      // (general instantiations: exactly one item, no loop)
+    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (strided and general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();
-    int lane = GENERAL ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    if (!GENERAL) asm volatile("" : "+v"(lane));
+    int lane = ONE_ITEM ? (int)threadIdx.x & 63 : (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (!ONE_ITEM) asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31;
     int bhk, kblock;
     fa_item_decode(item, a.B * a.Hk, n_kblocks, 0, &bhk, &kblock);
     const int b = bhk / a.Hk, hk = bhk - b * a.Hk;
-    const int q_rs = GENERAL ? a.q.rs : D, g_rs = GENERAL ? a.dO_.rs : D, k_rs = GENERAL ? a.k.rs : D, v_rs = GENERAL ? a.v.rs : D;
-    const int dk_rs = GENERAL ? a.dk.rs : D, dv_rs = GENERAL ? a.dv.rs : D;
+    const int q_rs = STRIDES ? a.q.rs : D, g_rs = STRIDES ? a.dO_.rs : D, k_rs = STRIDES ? a.k.rs : D, v_rs = STRIDES ? a.v.rs : D;
     const uint16_t *Kh, *Vh;
-    uint16_t *dKh, *dVh;
-    if (GENERAL) {
+    if (STRIDES) {
         Kh = head_ptr(a.K, a.k, b, hk); Vh = head_ptr(a.V, a.v, b, hk);
-        dKh = head_ptr(a.dK, a.dk, b, hk); dVh = head_ptr(a.dV, a.dv, b, hk);
     } else {
         const size_t head_off = (size_t)bhk * S * D;
-        Kh = a.K + head_off; Vh = a.V + head_off; dKh = a.dK + head_off; dVh = a.dV + head_off;
+        Kh = a.K + head_off; Vh = a.V + head_off;
     }
     const int k0 = kblock * 256, kw = k0 + wave * 32;
     const bool active = kw < Sk;
@@ -407,16 +419,22 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // Philox block covers sixteen keys of ONE query) reach the lanes that own the keys
     const uint32_t drop_lds = lds0 + kBwdStages * STAGEB + wave * 128;
     Loader ldq, ldg;
-    ldq.init(wave, lane, q_rs * 2);
+    if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);
     if (GENERAL) ldg.init(wave, lane, g_rs * 2);
     // g: query head inside the group of this K/V head
     auto issue = [&](int g, int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
         const int h = hk * G + g;
         const uint16_t *Qh, *dOh;
-        if (GENERAL) { Qh = head_ptr(a.Q, a.q, b, h); dOh = head_ptr(a.dO, a.dO_, b, h); }
-        else { Qh = a.Q + (size_t)bhk * S * D; dOh = a.dO + (size_t)bhk * S * D; }
-        const float *lse_h = a.lse2 + ((size_t)b * a.H + h) * S, *delta_h = a.delta + ((size_t)b * a.H + h) * S;
+        const float *lse_h, *delta_h;
+        if (STRIDES) {
+            const FaBwdArgs &f = args_reloaded();
+            Qh = head_ptr(f.Q, f.q, b, h); dOh = head_ptr(f.dO, f.dO_, b, h);
+            lse_h = f.lse2 + ((size_t)b * f.H + h) * S; delta_h = f.delta + ((size_t)b * f.H + h) * S;
+        } else {
+            Qh = a.Q + (size_t)bhk * S * D; dOh = a.dO + (size_t)bhk * S * D;
+            lse_h = a.lse2 + ((size_t)b * a.H + h) * S; delta_h = a.delta + ((size_t)b * a.H + h) * S;
+        }
         if (GENERAL && (tile + 1) * 64 > S) {
             const int valid = S - tile * 64;
             ldq.load_ragged(Qh + (size_t)tile * 64 * q_rs, base, valid, q_rs * 2);
@@ -425,9 +443,23 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             asm volatile("" : "+v"(ln));
             if (wave == 0) dma_4(lse_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB);
             if (wave == 1) dma_4(delta_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB + 256);
+        } else if (STRIDES && !GENERAL) {
+            // (the lanes' source offsets are formed here, from the hardware's lane index and freshly loaded strides:
+            // kept in registers from the top of the item they are spilled, and every reload in the tile loop waits
+            // for all loads in flight)
+            const FaBwdArgs &f = args_reloaded();
+            int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            asm volatile("" : "+v"(ln));
+            Loader lq, lg;
+            lq.init(wave, ln, f.q.rs * 2);
+            lg.init(wave, ln, f.dO_.rs * 2);
+            lq.load(Qh + (size_t)tile * 64 * f.q.rs, base);
+            lg.load(dOh + (size_t)tile * 64 * f.dO_.rs, base + TILEB);
+            if (wave == 0) dma_4(lse_h + tile * 64, ln, base + 2 * TILEB);
+            if (wave == 1) dma_4(delta_h + tile * 64, ln, base + 2 * TILEB + 256);
         } else {
             ldq.load(Qh + (size_t)tile * 64 * q_rs, base);
-            (GENERAL ? ldg : ldq).load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
+            (STRIDES ? ldg : ldq).load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
             if (wave == 0) dma_4(lse_h + tile * 64, lane, base + 2 * TILEB);
             if (wave == 1) dma_4(delta_h + tile * 64, lane, base + 2 * TILEB + 256);
         }
@@ -567,6 +599,15 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     asm volatile("" : "+v"(lane_e));
     const int key_e = kw + (lane_e & 31), half_e = lane_e >> 5;
     if (active && key_e < Sk) {
+        uint16_t *dKh, *dVh;
+        int dk_rs = D, dv_rs = D;
+        if (STRIDES) {
+            const FaBwdArgs &f = args_reloaded();
+            dKh = head_ptr(f.dK, f.dk, b, hk); dVh = head_ptr(f.dV, f.dv, b, hk);
+            dk_rs = f.dk.rs; dv_rs = f.dv.rs;
+        } else {
+            dKh = a.dK + (size_t)bhk * S * D; dVh = a.dV + (size_t)bhk * S * D;
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -583,15 +624,15 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     }   // next work item
 }
 
-template <bool BF16, int D, bool MASKED, bool GENERAL, bool ALIBI, bool DROPOUT>
+template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
 hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream)
 {
     constexpr int TILEB = 64 * D * 2;
     const unsigned grid_q = (unsigned)((long long)a.B * a.H * ((a.S + 255) / 256));
     const unsigned grid_k = (unsigned)((long long)a.B * a.Hk * ((a.Sk + 255) / 256));
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512) + (DROPOUT ? kBwdWaves * 128 : 0);
-    auto kq = fa_bwd_dq<BF16, D, MASKED, GENERAL, ALIBI, DROPOUT>;
-    auto kkv = fa_bwd_dkdv<BF16, D, MASKED, GENERAL, ALIBI, DROPOUT>;
+    auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
+    auto kkv = fa_bwd_dkdv<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
     const unsigned long long dev_bit = 1ull << fa_launch_device();
@@ -614,9 +655,10 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream)
     // (the general instantiations always carry the mask code: without a bound on either side, L = R = S + S_kv, their
     // items are alike as well)
     const long long unbounded = (long long)a.S + a.Sk;
-    // (The general instantiations are launched one workgroup per item only: with the item loop around them their
-    // 128-wide kernels spill ten times as much and run 15-20 % slower, c3's shape stored [B,S,H,D] 4.7 against 4.0 ms.)
-    const bool uneven = !GENERAL && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
+    // (The strided and general instantiations are launched one workgroup per item only: with the item loop around
+    // them their 128-wide kernels spill ten times as much, and a reload inside the tile loop waits for every tile
+    // load in flight: c3's shape stored [B,S,H,D] 4.1 ms against 3.8.)
+    const bool uneven = LAYOUT == 0 && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
     const unsigned launch_q = (uneven && grid_q > resident && grid_q < 16u * resident) ? resident : grid_q;
     const unsigned launch_k = (uneven && grid_k > resident && grid_k < 16u * resident) ? resident : grid_k;
     hipLaunchKernelGGL(kq, dim3(launch_q), dim3(kBwdWaves * 64), smem_dq, stream, a);

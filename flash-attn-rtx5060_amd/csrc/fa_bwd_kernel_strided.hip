@@ -1,0 +1,13 @@
+// Backward kernels for the strided layout: lengths as in the reference's layout (S a multiple of 128, as many
+// keys), any row, head and batch strides, grouped K/V heads; in a translation unit of their own.
+#include "fa_bwd_kernel_impl.h"
+
+hipError_t fa_launch_backward_strided(const FaBwdArgs &a, int bf16, int D, int masked, int compute_units, hipStream_t stream)
+{
+#define FA_BWD_CASE(BF, DD, MK) \
+    if (bf16 == BF && D == DD && masked == MK) return launch_bwd<BF != 0, DD, MK != 0, 1, false, false>(a, compute_units, stream);
+    FA_BWD_CASE(0, 64, 0) FA_BWD_CASE(0, 64, 1) FA_BWD_CASE(0, 128, 0) FA_BWD_CASE(0, 128, 1)
+    FA_BWD_CASE(1, 64, 0) FA_BWD_CASE(1, 64, 1) FA_BWD_CASE(1, 128, 0) FA_BWD_CASE(1, 128, 1)
+#undef FA_BWD_CASE
+    return hipErrorInvalidValue;
+}

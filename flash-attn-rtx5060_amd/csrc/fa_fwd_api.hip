@@ -32,6 +32,7 @@ hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipS
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, int compute_units,
                               hipStream_t stream);
 hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream);
+hipError_t fa_launch_backward_strided(const FaBwdArgs &a, int bf16, int D, int masked, int compute_units, hipStream_t stream);
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -595,7 +596,9 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.Hk = p->n_kv_heads > 0 ? p->n_kv_heads : p->N;
     a.S = p->S;
     a.Sk = p->S_kv > 0 ? p->S_kv : p->S;
-    bool general = a.Hk != a.H || a.S % 128 != 0 || a.Sk != a.S || a.alibi != nullptr;
+    // general: any lengths, ALiBi, dropout; strided: the reference's lengths with other strides or grouped K/V heads
+    const bool general = a.S % 128 != 0 || a.Sk != a.S || a.alibi != nullptr;
+    bool strided = a.Hk != a.H;
     {
         const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
                                        p->dq_strides, p->dk_strides, p->dv_strides};
@@ -609,7 +612,7 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
             long long eff[3];
             for (int k = 0; k < 3; ++k) {
                 eff[k] = given ? st[k] : dense[k];
-                if (eff[k] != dense[k]) general = true;
+                if (eff[k] != dense[k]) strided = true;
             }
             out[t]->bs = eff[0]; out[t]->hs = eff[1]; out[t]->rs = (int)eff[2];
         }
@@ -626,7 +629,9 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     hipError_t e = a.drop_threshold != 0
         ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, ds->compute_units,
                                      static_cast<hipStream_t>(stream))
-        : fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general ? 1 : 0, a.alibi != nullptr ? 1 : 0,
+        : (strided && !general)
+        ? fa_launch_backward_strided(a, p->dtype == FA_DTYPE_BF16, p->d, masked, ds->compute_units, static_cast<hipStream_t>(stream))
+        : fa_launch_backward(a, p->dtype == FA_DTYPE_BF16, p->d, masked, general || strided ? 1 : 0, a.alibi != nullptr ? 1 : 0,
                              ds->compute_units, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? FA_OK : device_fail(e, "backward launch");
 }

@@ -127,6 +127,11 @@ GENERAL = [
     (1, 2, 2, 1, 500, 128, 0, True, -1, -1, False, False),         # a single query
     (1, 2, 1, 300, 300, 128, 0, True, -1, -1, False, False),
     (1, 2, 2, 256, 256, 64, 0, True, -1, -1, True, False),         # ALiBi on a shape the plain kernels cover
+    # the reference's lengths with other strides or grouped heads: the strided kernels
+    (2, 4, 2, 512, 512, 128, 0, True, -1, -1, False, True),
+    (1, 4, 4, 384, 384, 64, 1, True, 100, -1, False, True),
+    (1, 6, 2, 256, 256, 64, 0, False, -1, -1, False, False),
+    (1, 2, 1, 640, 640, 128, 1, False, 64, 64, False, True),
 ]
 
 
@@ -150,6 +155,26 @@ def test_general_layouts_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D
         err = grad_errors(oracle.to_f32(from_torch(got.contiguous()), dtype), want)
         print((B, H, Hk, S, Skv, D), dtype, causal, wl, wr, alibi, bshd, name, err, flush=True)
         check(err, dtype, name)
+
+
+@pytest.mark.parametrize("D,dtype,causal,wl", [(128, 0, True, -1), (64, 1, False, -1), (128, 1, True, 200), (64, 0, True, -1)])
+def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl):
+    """[B,S,H,D] storage goes through the strided kernels, [B,H,S,D] through the plain ones: same values, same
+    arithmetic in the same order, so dQ, dK and dV have to agree bit for bit."""
+    import torch
+    B, H, S = 2, 3, 768
+    q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed=910 + D)
+    do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=911 + D)
+    dense = [to_torch(x, dtype) for x in (q, k, v, do)]
+    bshd = [t.transpose(1, 2).contiguous().transpose(1, 2) for t in dense]
+    got = []
+    for tq, tk, tv, tdo in (dense, bshd):
+        o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl)
+        got.append(fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl))
+    torch.cuda.synchronize()
+    assert got[1][0].stride() == bshd[0].stride()
+    for name, a, b in zip(("dQ", "dK", "dV"), got[0], got[1]):
+        assert torch.equal(a.view(torch.int16), b.contiguous().view(torch.int16)), name
 
 
 def test_queries_without_any_key_get_zero_gradients(fa):
