@@ -126,7 +126,9 @@ def backward_bench(args):
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
     if args.layout == "bshd":
         tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
-    kw = dict(causal=causal, window_left=wl, dropout_prob=args.dropout, seed=48)
+    slopes = np.power(2.0, -8.0 / H * (np.arange(H) + 1)).astype(np.float32) if args.alibi else None
+    kw = dict(causal=causal, window_left=wl, dropout_prob=args.dropout, seed=48,
+              alibi_slopes=torch.from_numpy(slopes).cuda() if args.alibi else None)
     o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
     grads = [None]
 
@@ -154,6 +156,8 @@ def backward_bench(args):
     if wl >= 0:
         vis &= i[:, None] - i[None, :] <= wl
     sc = (qf @ kf.T) * float(np.float32(1.0 / np.sqrt(D)))
+    if args.alibi:
+        sc = sc - float(slopes[-1]) * (i[:, None] - i[None, :]).abs().float()
     pm = torch.softmax(sc.masked_fill(~vis, float("-inf")), dim=-1)
     if args.dropout > 0:
         from parity_util import numpy_keep_mask
@@ -171,13 +175,13 @@ def backward_bench(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if dtype else "fp16", "data": "synthetic",
         "config": {"workload": f"{args.workload} backward: {'bf16' if dtype else 'fp16'} B{B} H{H} S{S} D{D}"
                                f"{' causal' if causal else ''}{f' window_left {wl}' if wl >= 0 else ''}"
-                               f"{f' dropout {args.dropout}' if args.dropout > 0 else ''}"
+                               f"{', ALiBi' if args.alibi else ''}{f' dropout {args.dropout}' if args.dropout > 0 else ''}"
                                f"{', stored [B,S,H,D]' if args.layout == 'bshd' else ''}"
                                f"{f', {args.kv_heads} K/V heads' if args.kv_heads else ''}",
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads else None,
+                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads and not args.alibi else None,
                      "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_dq + fa_bwd_dkdv"},
         "parity_vs_torch_fp32_one_head": err}))
 

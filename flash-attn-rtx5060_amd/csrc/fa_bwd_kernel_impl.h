@@ -419,7 +419,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // Philox block covers sixteen keys of ONE query) reach the lanes that own the keys
     const uint32_t drop_lds = lds0 + kBwdStages * STAGEB + wave * 128;
     Loader ldq, ldg;
-    if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);
+    if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);      // (general: only its ragged tiles go through these two)
     if (GENERAL) ldg.init(wave, lane, g_rs * 2);
     // g: query head inside the group of this K/V head
     auto issue = [&](int g, int tile, int stage) __attribute__((always_inline)) {
@@ -443,7 +443,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             asm volatile("" : "+v"(ln));
             if (wave == 0) dma_4(lse_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB);
             if (wave == 1) dma_4(delta_h + tile * 64, ln < valid ? ln : valid - 1, base + 2 * TILEB + 256);
-        } else if (STRIDES && !GENERAL) {
+        } else if (STRIDES) {
             // (the lanes' source offsets are formed here, from the hardware's lane index and freshly loaded strides:
             // kept in registers from the top of the item they are spilled, and every reload in the tile loop waits
             // for all loads in flight)
@@ -459,7 +459,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             if (wave == 1) dma_4(delta_h + tile * 64, ln, base + 2 * TILEB + 256);
         } else {
             ldq.load(Qh + (size_t)tile * 64 * q_rs, base);
-            (STRIDES ? ldg : ldq).load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
+            ldq.load(dOh + (size_t)tile * 64 * g_rs, base + TILEB);
             if (wave == 0) dma_4(lse_h + tile * 64, lane, base + 2 * TILEB);
             if (wave == 1) dma_4(delta_h + tile * 64, lane, base + 2 * TILEB + 256);
         }
