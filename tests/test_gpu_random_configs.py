@@ -86,11 +86,12 @@ def test_random_configurations(fa, regular):
         o_ref, lse_ref, dq_ref, dk_ref, dv_ref = reference(q, k, v, do, causal, wl, wr, slopes, keep)
         half = dtype == torch.float16
         assert bool(torch.isfinite(o.float()).all()), what
-        # the tolerance, or one ulp of the storage type where a row of few keys makes the output so large
-        # (|O| >= 4) that one ulp exceeds it: p and the result are each rounded once to the storage type
+        # the tolerance, or one and a half ulps of the storage type where a row of few keys makes the output so
+        # large that they exceed it: p and the result are each rounded once to the storage type, which puts the
+        # result up to one step beside the rounded reference, itself up to half a step from the exact one
         # (an indexing mistake shows up as an error of order one)
         one_ulp = torch.exp2(torch.floor(torch.log2(o_ref.abs().clamp_min(1e-4))) - (10 if half else 7))
-        bound = torch.maximum(one_ulp, torch.full_like(one_ulp, 2e-3 if half else 1.6e-2)) * grow
+        bound = torch.maximum(1.5 * one_ulp, torch.full_like(one_ulp, 2e-3 if half else 1.6e-2)) * grow
         assert bool(((o.float() - o_ref).abs() <= bound).all()), (what, float((o.float() - o_ref).abs().max()))
         seen = torch.isfinite(lse_ref)
         assert bool((lse[~seen] == float("-inf")).all()), what
@@ -101,4 +102,6 @@ def test_random_configurations(fa, regular):
             scale = max(1.0, float(want.abs().max()))
             assert bool(torch.isfinite(got.float()).all()), (name, what)
             assert float(d.abs().max()) <= (2e-3 if half else 1.6e-2) * scale * grow, (name, float(d.abs().max()), what)
-            assert float(d.norm()) <= (1e-3 if half else 8e-3) * grow * float(want.norm()) + 1e-5, (name, what)
+            # (plus 1e-5 per element: under a window of one key dS = P (dP - delta) is zero in exact arithmetic, and the
+            # kernels' dP and delta are the same sum taken in two orders, so dQ and dK come out as a few 1e-6)
+            assert float(d.norm()) <= (1e-3 if half else 8e-3) * grow * float(want.norm()) + 1e-5 * want.numel() ** 0.5, (name, what)
