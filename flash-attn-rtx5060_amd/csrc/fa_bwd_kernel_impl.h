@@ -422,15 +422,24 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);      // (general: only its ragged tiles go through these two)
     if (GENERAL) ldg.init(wave, lane, g_rs * 2);
     // g: query head inside the group of this K/V head
+    // strided layouts: where the walked query head starts (Q, dO, its rescaled logsumexps and deltas), formed when the
+    // walk moves to the next head of the group and carried in eight scalar registers; the strides themselves are
+    // read again at every fetch
+    const uint16_t *walk_q = nullptr, *walk_g = nullptr;
+    const float *walk_lse = nullptr, *walk_delta = nullptr;
+    auto walk_head = [&](int g) __attribute__((always_inline)) {
+        const FaBwdArgs &f = args_reloaded();
+        const int h = hk * G + g;
+        walk_q = head_ptr(f.Q, f.q, b, h); walk_g = head_ptr(f.dO, f.dO_, b, h);
+        walk_lse = f.lse2 + ((size_t)b * f.H + h) * S; walk_delta = f.delta + ((size_t)b * f.H + h) * S;
+    };
     auto issue = [&](int g, int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
         const int h = hk * G + g;
         const uint16_t *Qh, *dOh;
         const float *lse_h, *delta_h;
         if (STRIDES) {
-            const FaBwdArgs &f = args_reloaded();
-            Qh = head_ptr(f.Q, f.q, b, h); dOh = head_ptr(f.dO, f.dO_, b, h);
-            lse_h = f.lse2 + ((size_t)b * f.H + h) * S; delta_h = f.delta + ((size_t)b * f.H + h) * S;
+            Qh = walk_q; dOh = walk_g; lse_h = walk_lse; delta_h = walk_delta;
         } else {
             Qh = a.Q + (size_t)bhk * S * D; dOh = a.dO + (size_t)bhk * S * D;
             lse_h = a.lse2 + ((size_t)b * a.H + h) * S; delta_h = a.delta + ((size_t)b * a.H + h) * S;
@@ -561,8 +570,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
         int ig = 0, it = t1;                                    // the next pair to fetch
         auto issue_next = [&](int stage) __attribute__((always_inline)) {
             issue(ig, it, stage);
-            if (--it < t0) { it = t1; ++ig; }
+            if (--it < t0) {
+                it = t1; ++ig;
+                if (STRIDES && ig < G) walk_head(ig);
+            }
         };
+        if (STRIDES) walk_head(0);
         issue_next(0);
         if (ig < G) issue_next(1);
         wait_vm<0>();
