@@ -396,7 +396,6 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     const bool active = kw < Sk;
     const int my_k = kw + l32;                     // this lane's key (masks, ALiBi)
     const int my_kc = active ? (GENERAL && my_k >= Sk ? Sk - 1 : my_k) : (GENERAL ? 0 : l32);     // row to load
-    const bool row_ok = active && my_k < Sk;
 
     u32x4 kf[KS], vf[KS];           // K^T and V^T as B operands: lane = (key, head-dim slice)
 #pragma unroll
@@ -421,7 +420,6 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     Loader ldq, ldg;
     if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);      // (general: only its ragged tiles go through these two)
     if (GENERAL) ldg.init(wave, lane, g_rs * 2);
-    // g: query head inside the group of this K/V head
     // strided layouts: where the walked query head starts (Q, dO, its rescaled logsumexps and deltas), formed when the
     // walk moves to the next head of the group and carried in eight scalar registers; the strides themselves are
     // read again at every fetch
@@ -433,6 +431,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
         walk_q = head_ptr(f.Q, f.q, b, h); walk_g = head_ptr(f.dO, f.dO_, b, h);
         walk_lse = f.lse2 + ((size_t)b * f.H + h) * S; walk_delta = f.delta + ((size_t)b * f.H + h) * S;
     };
+    // g: query head inside the group of this K/V head
     auto issue = [&](int g, int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
         const int h = hk * G + g;
