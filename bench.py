@@ -253,6 +253,25 @@ def main():
         fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, out=out, lse=lse, sched=args.sched,
                                    alibi_slopes=tslopes, dropout_prob=args.dropout, seed=48)
 
+    def timed(n_warmup, n_steps):
+        # exactly n_steps launches back to back, one HIP event on the launch stream in front of the first and one
+        # behind the last (an event between two launches is a packet of its own and costs a 60 us kernel 4 us of
+        # gap); the kernel's average duration is the events' distance over the number of launches
+        for _ in range(n_warmup):
+            step()
+        torch.cuda.synchronize()
+        e_first, e_last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e_first.record()
+        for _ in range(n_steps):
+            step()
+        e_last.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n_steps, e_first.elapsed_time(e_last) / n_steps
+
+    # The same protocol without the clock-settle phase, on the still idle chip (reported next to the headline as
+    # `without_settle`, so that figures taken with and without the phase can be compared like for like).
+    cold_wall_ms, cold_kernel_ms = timed(args.warmup, args.steps) if args.settle_ms > 0 else (None, None)
     # clock settle (untimed, reported): launches back to back until the wall clock says settle_ms have passed
     settle_steps = 0
     if args.settle_ms > 0:
@@ -262,21 +281,7 @@ def main():
                 step()
             settle_steps += 8
             torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # the timed region: exactly `steps` launches back to back, one HIP event on the launch stream in front of the
-    # first and one behind the last (an event between two launches is a packet of its own and costs a 60 us
-    # kernel 4 us of gap); the kernel's average duration is the events' distance over the number of launches
-    e_first, e_last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e_first.record()
-    for i in range(args.steps):
-        step()
-    e_last.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    avg_kernel_ms = e_first.elapsed_time(e_last) / args.steps
+    wall_ms, avg_kernel_ms = timed(args.warmup, args.steps)        # the timed region of the headline figure
     # (a second, untimed pass with an event after every launch, for the spread only)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     ev[0].record()
@@ -322,6 +327,11 @@ def main():
                      "kernel_ms_min": round(float(np.min(kernel_ms)), 5),
                      "kernel_ms_avg_from": "two events around the timed launches", "kernel_ms_median_min_from": "a second pass with an event after every launch"},
     }
+    if cold_wall_ms is not None:
+        result["without_settle"] = {"value": round(flops / (cold_wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(cold_wall_ms, 5),
+                                    "kernel_ms_avg": round(cold_kernel_ms, 5),
+                                    "frac": round(flops / (cold_kernel_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4),
+                                    "note": "same steps and warm-up, run first, before the clock-settle phase"}
 
     drop = (fa.lib().fa_dropout_threshold(args.dropout), 48)
     rep = H // k.shape[1]
@@ -348,15 +358,17 @@ def main():
         t = time.perf_counter()
         ob.rows(q, kf, vf, probe, dtype, None, causal, wl, -1, slopes, threads=cores, dropout=drop)
         per_row = max((time.perf_counter() - t) / len(probe), 1e-7)
-        n = int(min(B * H * S, max(len(probe), args.cpu_seconds / per_row)))
-        for attempt in range(2):    # (the probe overestimates the cost per row: one resize if the sample came out short)
+        n = int(min(B * H * S, max(len(probe), 0.5 * args.cpu_seconds / per_row)))
+        spent = 0.0
+        for attempt in range(2):    # (one resize if the first sample came out short; both together stay near the target)
             sample = np.sort(rng.choice(B * H * S, size=n, replace=False))
             t = time.perf_counter()
             ob.rows(q, kf, vf, sample, dtype, None, causal, wl, -1, slopes, threads=cores, dropout=drop)
             dt = time.perf_counter() - t
-            if dt >= 0.6 * args.cpu_seconds or n >= B * H * S:
+            spent += dt
+            if dt >= 0.4 * args.cpu_seconds or n >= B * H * S:
                 break
-            n = int(min(B * H * S, n * args.cpu_seconds / max(dt, 1e-3)))
+            n = int(min(B * H * S, n * max(args.cpu_seconds - spent, 0.0) / max(dt, 1e-3)))
         pairs = 0
         for r in sample.tolist():
             i = r % S
@@ -366,8 +378,10 @@ def main():
         cpu_tflops = 4.0 * D * pairs / dt / 1e12
         result["cpu_baseline"] = {
             "value": round(cpu_tflops, 5), "unit": "TFLOPS", "cores": cores, "kind": "port",
-            "sample": f"{'all ' if n >= B * H * S else ''}{n} {'' if n >= B * H * S else 'uniformly sampled '}query rows of the same workload ({pairs} unmasked pairs), "
-                      f"{dt:.1f} s on {cores} threads; extrapolated whole problem: {flops / (cpu_tflops * 1e12):.0f} s",
+            "sample": (f"all {n} query rows of the same workload ({pairs} unmasked pairs): the whole problem, {dt:.1f} s on {cores} threads"
+                       if n >= B * H * S else
+                       f"{n} uniformly sampled query rows of the same workload ({pairs} unmasked pairs), {dt:.1f} s on {cores} threads; "
+                       f"at that rate the whole problem would take {flops / (cpu_tflops * 1e12):.0f} s"),
         }
     print(json.dumps(result))
 

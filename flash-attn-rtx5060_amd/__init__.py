@@ -46,7 +46,7 @@ FA_TILE_SKIP, FA_TILE_PARTIAL, FA_TILE_FULL = 0, 1, 2
 #: every symbol include/fa_fwd.h declares
 EXPORTED_SYMBOLS = (
     "fa_fwd_validate", "fa_fwd", "fa_init", "fa_fwd_split_static", "fa_fwd_static_scratch_bytes",
-    "fa_reset_work_queues", "run_flash_attention", "fa_strerror", "fa_last_device_error",
+    "fa_reset_work_queues", "fa_release_work_queue", "run_flash_attention", "fa_strerror", "fa_last_device_error",
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_heads", "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
@@ -130,6 +130,7 @@ def lib():
         L.fa_fwd.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
         L.fa_fwd_split_static.argtypes = [ctypes.POINTER(FaFwdParams), ctypes.c_void_p]
         L.fa_fwd_static_scratch_bytes.restype = ctypes.c_ulonglong
+        L.fa_release_work_queue.argtypes = [ctypes.c_void_p]
         L.fa_fwd_workspace_bytes.restype = ctypes.c_ulonglong
         L.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.fa_fwd_suggest_splits.argtypes = [ctypes.POINTER(FaFwdParams)]

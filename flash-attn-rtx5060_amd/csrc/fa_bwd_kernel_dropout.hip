@@ -1,12 +1,26 @@
 // Backward kernels with dropout (general layout, with and without ALiBi), in a translation unit of their own.
 #include "fa_bwd_kernel_impl.h"
 
-hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream)
+hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream,
+                                      bool configure_only)
 {
 #define FA_BWD_CASE(BF, DD, AL) \
-    if (bf16 == BF && D == DD && alibi == AL) return launch_bwd<BF != 0, DD, true, 2, AL != 0, true>(a, compute_units, stream);
+    if (bf16 == BF && D == DD && alibi == AL) return launch_bwd<BF != 0, DD, true, 2, AL != 0, true>(a, compute_units, stream, configure_only);
     FA_BWD_CASE(0, 64, 0) FA_BWD_CASE(0, 128, 0) FA_BWD_CASE(1, 64, 0) FA_BWD_CASE(1, 128, 0)
     FA_BWD_CASE(0, 64, 1) FA_BWD_CASE(0, 128, 1) FA_BWD_CASE(1, 64, 1) FA_BWD_CASE(1, 128, 1)
 #undef FA_BWD_CASE
     return hipErrorInvalidValue;
+}
+
+// the LDS opt-in of every instantiation above for the current device, without a launch (fa_init)
+hipError_t fa_configure_backward_dropout()
+{
+    const FaBwdArgs a = {};
+    for (int bf16 = 0; bf16 < 2; ++bf16)
+        for (int D = 64; D <= 128; D += 64)
+            for (int alibi = 0; alibi < 2; ++alibi) {
+                const hipError_t e = fa_launch_backward_dropout(a, bf16, D, alibi, 0, nullptr, true);
+                if (e != hipSuccess) return e;
+            }
+    return hipSuccess;
 }

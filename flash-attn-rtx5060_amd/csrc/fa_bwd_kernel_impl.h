@@ -637,7 +637,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
 }
 
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
-hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream)
+hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream, bool configure_only = false)
 {
     constexpr int TILEB = 64 * D * 2;
     const unsigned grid_q = (unsigned)((long long)a.B * a.H * ((a.S + 255) / 256));
@@ -655,6 +655,7 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream)
         if (e != hipSuccess) return e;
         configured.fetch_or(dev_bit, std::memory_order_relaxed);
     }
+    if (configure_only) return hipSuccess;     // (fa_init: the opt-in alone, so that no launch inside a stream capture makes it)
     // Masked problems with between one and sixteen items per compute unit: a resident grid (one workgroup per CU,
     // 8 waves at two per SIMD) walks the list as a snake, which pairs every long item with a short one; otherwise
     // one workgroup per item, handed out by the hardware as CUs free up.  Causal fp16, snake against dispatch:

@@ -6,6 +6,7 @@
 // exits, aborts or throws, launches asynchronously on the caller's stream,
 // keeps no global descriptor state, and does not time or print.
 #include <hip/hip_runtime.h>
+#include <dlfcn.h>
 #include <math.h>
 #include <stdio.h>
 #include <string.h>
@@ -30,9 +31,19 @@ hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int
                                      hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, int compute_units,
-                              hipStream_t stream);
-hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream);
-hipError_t fa_launch_backward_strided(const FaBwdArgs &a, int bf16, int D, int masked, int compute_units, hipStream_t stream);
+                              hipStream_t stream, bool configure_only = false);
+hipError_t fa_launch_backward_dropout(const FaBwdArgs &a, int bf16, int D, int alibi, int compute_units, hipStream_t stream,
+                                      bool configure_only = false);
+hipError_t fa_launch_backward_strided(const FaBwdArgs &a, int bf16, int D, int masked, int compute_units, hipStream_t stream,
+                                      bool configure_only = false);
+// the LDS opt-in (hipFuncSetAttribute) of every kernel instantiation of a translation unit, for the current device
+hipError_t fa_configure_forward_contiguous();
+hipError_t fa_configure_forward_strided();
+hipError_t fa_configure_forward_general();
+hipError_t fa_configure_forward_dropout();
+hipError_t fa_configure_backward();
+hipError_t fa_configure_backward_dropout();
+hipError_t fa_configure_backward_strided();
 
 namespace {
 constexpr int kBlockKeysHost = 64;
@@ -51,35 +62,61 @@ int waves_for(int B, int N, int S)
 thread_local char g_last_error[256] = "";
 
 std::atomic<unsigned> g_capture_ticket[kFaMaxDevices];     // captured queue launches so far, per device
-// eager launches: which stream owns which counter set of a device (0 = free; the legacy default stream is kept as 1)
-std::atomic<uintptr_t> g_slot_owner[kFaMaxDevices][kFaEagerQueueSlots];
+// Eager launches: which stream owns which counter set of a device.  A stream is named by its handle AND the id
+// the runtime gave it at creation (hipStreamGetId): a handle value can come back for a new stream after the old
+// one was destroyed, while the old stream's last launch may still be running on its counters; the id never does.
+struct SlotOwner {
+    uintptr_t handle;           // 0 = free
+    unsigned long long id;
+};
+std::mutex g_slot_mutex;
+// hipStreamGetId exists from HIP 7.1 on; a process may have loaded an older runtime (PyTorch wheels bring their
+// own), so it is looked up at run time.  Without it a stream is named by its handle alone, and a caller that
+// destroys streams has to release their sets first (fa_release_work_queue).
+typedef hipError_t (*StreamIdFn)(hipStream_t, unsigned long long *);
+bool stream_id(hipStream_t stream, unsigned long long *id)
+{
+    static const StreamIdFn fn = reinterpret_cast<StreamIdFn>(dlsym(RTLD_DEFAULT, "hipStreamGetId"));
+    *id = 0;
+    return fn == nullptr || fn(stream, id) == hipSuccess;
+}
+SlotOwner g_slot_owner[kFaMaxDevices][kFaEagerQueueSlots];
 
 // A counter set for one FA_SCHED_QUEUE launch, or null when none can be given safely (the caller then walks the
-// list with the fixed snake).  Eager launches: a set belongs to a stream -- launches on one stream run one after
-// the other, so they may share it, and every launch leaves it rewound; a device hands out sixteen sets, to the
-// first sixteen streams that ask (a stream keeps its set for the life of the process), and further streams get
-// none.  A launch that is being captured into a graph keeps its set for every replay of that graph, and a replay
-// may run next to anything: every captured launch gets a set of its own from the remaining 240, for good, and
-// when those are used up captured launches get none.  No two launches that can run at the same time ever share
-// counters.
+// list with the fixed snake: same results, no counters).  Eager launches: a set belongs to a stream -- launches on
+// one stream run one after the other, so they may share it, and every launch leaves it rewound; a device hands out
+// sixteen sets, to the first sixteen streams that ask, and a stream keeps its set until fa_release_work_queue or
+// fa_reset_work_queues; further streams get none.  hipStreamPerThread gets none either: it is one handle value
+// for a different stream in every host thread.  A launch that is being captured into a graph keeps its set for
+// every replay of that graph, and a replay may run next to anything: every captured launch gets a set of its own
+// from the remaining 240, for good, and when those are used up captured launches get none.  No two launches that
+// can run at the same time ever share counters.
 unsigned *work_queue_for_launch(const FaDeviceState *ds, hipStream_t stream)
 {
+    if (stream == hipStreamPerThread) return nullptr;
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    const bool capturing = stream != nullptr && hipStreamIsCapturing(stream, &status) == hipSuccess &&
+    const bool capturing = stream != nullptr && stream != hipStreamLegacy && hipStreamIsCapturing(stream, &status) == hipSuccess &&
                            status == hipStreamCaptureStatusActive;
     if (capturing) {
         const unsigned n = g_capture_ticket[fa_launch_device()].fetch_add(1u, std::memory_order_relaxed);
         if (n >= (unsigned)(kFaQueueSlots - kFaEagerQueueSlots)) return nullptr;
         return ds->queues + 16u * ((unsigned)kFaEagerQueueSlots + n);
     }
-    const uintptr_t key = stream == nullptr ? (uintptr_t)1 : reinterpret_cast<uintptr_t>(stream);
-    std::atomic<uintptr_t> *owners = g_slot_owner[fa_launch_device()];
-    for (unsigned i = 0; i < (unsigned)kFaEagerQueueSlots; ++i) {
-        uintptr_t seen = owners[i].load(std::memory_order_acquire);
-        if (seen == 0 && owners[i].compare_exchange_strong(seen, key, std::memory_order_acq_rel)) seen = key;
-        if (seen == key) return ds->queues + 16u * i;
+    // (the two names of the legacy default stream are one stream)
+    const bool legacy = stream == nullptr || stream == hipStreamLegacy;
+    const uintptr_t handle = legacy ? (uintptr_t)1 : reinterpret_cast<uintptr_t>(stream);
+    unsigned long long id = 0;
+    if (!legacy && !stream_id(stream, &id)) return nullptr;
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    SlotOwner *owners = g_slot_owner[fa_launch_device()];
+    int free_slot = -1;
+    for (int i = 0; i < kFaEagerQueueSlots; ++i) {
+        if (owners[i].handle == handle && owners[i].id == id) return ds->queues + 16u * (unsigned)i;
+        if (owners[i].handle == 0 && free_slot < 0) free_slot = i;
     }
-    return nullptr;
+    if (free_slot < 0) return nullptr;
+    owners[free_slot] = SlotOwner{handle, id};
+    return ds->queues + 16u * (unsigned)free_slot;
 }
 
 int device_fail(hipError_t e, const char *what)
@@ -412,8 +449,18 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
 int fa_init(void)
 {
     const FaDeviceState *ds = nullptr;
-    const hipError_t e = fa_device_state(&ds);
-    return e == hipSuccess ? FA_OK : device_fail(e, "device set-up");
+    hipError_t e = fa_device_state(&ds);
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    // everything a first launch would otherwise do besides the launch itself: after this call no entry point makes
+    // a HIP call on this device that is not a stream operation (which is what a stream capture needs)
+    hipError_t (*const configure[])() = {fa_configure_forward_contiguous, fa_configure_forward_strided, fa_configure_forward_general,
+                                         fa_configure_forward_dropout, fa_configure_backward, fa_configure_backward_dropout,
+                                         fa_configure_backward_strided};
+    for (auto fn : configure) {
+        e = fn();
+        if (e != hipSuccess) return device_fail(e, "kernel set-up");
+    }
+    return FA_OK;
 }
 
 int fa_fwd(const fa_fwd_params *p, void *stream)
@@ -450,7 +497,29 @@ int fa_reset_work_queues(void)
     e = hipMemset(ds->queues, 0, (size_t)kFaQueueSlots * 16 * sizeof(unsigned));
     if (e != hipSuccess) return device_fail(e, "work queue reset");
     // (nothing is in flight after the synchronisation: streams may claim their sets anew)
-    for (int i = 0; i < kFaEagerQueueSlots; ++i) g_slot_owner[fa_launch_device()][i].store(0, std::memory_order_release);
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    for (int i = 0; i < kFaEagerQueueSlots; ++i) g_slot_owner[fa_launch_device()][i] = SlotOwner{0, 0};
+    return FA_OK;
+}
+
+int fa_release_work_queue(void *stream_handle)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+    const FaDeviceState *ds = nullptr;
+    hipError_t e = fa_device_state(&ds);
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    if (stream == hipStreamPerThread) return FA_OK;             // never owns a set
+    const bool legacy = stream == nullptr || stream == hipStreamLegacy;
+    const uintptr_t handle = legacy ? (uintptr_t)1 : reinterpret_cast<uintptr_t>(stream);
+    unsigned long long id = 0;
+    if (!legacy && !stream_id(stream, &id)) return device_fail(hipErrorInvalidHandle, "hipStreamGetId");
+    // the stream's last launch must have left the set rewound before another stream may take it
+    e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return device_fail(e, "synchronize");
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    SlotOwner *owners = g_slot_owner[fa_launch_device()];
+    for (int i = 0; i < kFaEagerQueueSlots; ++i)
+        if (owners[i].handle == handle && owners[i].id == id) owners[i] = SlotOwner{0, 0};
     return FA_OK;
 }
 

@@ -58,11 +58,4 @@ hipError_t fa_launch_forward_contiguous(const FaKernelArgs &a, int bf16, int D, 
 {
     return launch_forward<false, false>(a, bf16, D, masked, shape, grid, stream);
 }
-
-#ifdef FA_TIMELINE
-// working aid (see fa_fwd_kernel_impl.h): sets the buffer the contiguous-layout kernels write their timeline to
-extern "C" int fa_debug_set_timeline(long long *device_buffer)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_fa_timeline), &device_buffer, sizeof(device_buffer));
-}
-#endif
+hipError_t fa_configure_forward_contiguous() { return configure_forward<false, false>(); }

@@ -6,3 +6,4 @@ hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int
 {
     return launch_forward<true, true>(a, bf16, D, masked, shape, grid, stream);
 }
+hipError_t fa_configure_forward_dropout() { return configure_forward<true, true>(); }

@@ -7,6 +7,7 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
 {
     return launch_forward<true, false>(a, bf16, D, masked, shape, grid, stream);
 }
+hipError_t fa_configure_forward_general() { return configure_forward<true, false>(); }
 
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream)
 {

@@ -89,36 +89,6 @@ template <> struct Num<true> {
     }
 };
 
-// The same matrix instructions with their register files pinned, for the 64-rows-per-wave shape (one wave per
-// SIMD, 512 registers): the O^T accumulators and the Q^T fragments live in the accumulation registers, which
-// only matrix instructions touch, the S^T accumulators and everything the vector ALU works on in the ordinary
-// ones.  Left to the register allocator, values wander between the two files (about 240 moves per tile).
-// Written as inline assembly the compiler no longer sees a matrix instruction and inserts no wait states for
-// it: every place where a result is read by a vector instruction within about twenty cycles carries an
-// explicit s_nop (mfma_result_wait), and results are reused as accumulators only several matrix
-// instructions later.
-template <bool BF16> struct PinnedMfma {
-    // S^T block: D in ordinary registers, B operand (Q^T) in accumulation registers; first of a chain: C = 0
-    static __device__ __forceinline__ void qk_first(f32x16 &d, u32x4 a, u32x4 b)
-    {
-        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
-        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
-    }
-    static __device__ __forceinline__ void qk_next(f32x16 &d, u32x4 a, u32x4 b)
-    {
-        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-    }
-    // O^T block: accumulator in accumulation registers, operands in ordinary registers
-    static __device__ __forceinline__ void pv(f32x16 &acc, u32x4 a, u32x4 b)
-    {
-        if (BF16) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-    }
-};
-// wait states between a pinned matrix instruction and a vector instruction that reads its result
-__device__ __forceinline__ void mfma_result_wait() { asm volatile("s_nop 15\n\ts_nop 9" ::: "memory"); }
-
 // 16-byte-chunk swizzles.  A tile row holds CPR = D/8 chunks.
 // K is read with ds_read_b128 by 16 lanes holding 16 consecutive rows and one
 // logical chunk: those must land on 16 different 16-byte bank groups.
@@ -178,18 +148,6 @@ __device__ __forceinline__ void dma_16(const char *base, uint32_t voff, uint32_t
 __device__ __forceinline__ void phase_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int V> struct IntC { static constexpr int value = V; };
-
-// Per-item timeline for performance work: compiled only with -DFA_TIMELINE (never in the shipped library).
-// Thread 0 of every workgroup writes sixteen 64-bit words per work item: item, XCD and CU id, then the 100 MHz
-// wall clock when the item was taken, after the prologue, after the tile loop, after the epilogue, after
-// the first-rows path, the numbers of fill+drain and steady iterations, the tile range, and (words 10-14) the
-// shader clock counter at the same five points.
-#ifdef FA_TIMELINE
-__device__ long long *g_fa_timeline = nullptr;
-#define FA_TL(slot) do { if (tid == 0) { tl_lds[slot] = (long long)__builtin_amdgcn_s_memrealtime(); tl_lds[slot + 8] = (long long)__builtin_amdgcn_s_memtime(); } } while (0)
-#else
-#define FA_TL(slot) do { } while (0)
-#endif
 
 // ---------------------------------------------------------------------------
 // First rows of a causal head, in the reference's own arithmetic.
@@ -425,19 +383,17 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 }
 
 // ---------------------------------------------------------------------------
-// The kernel.  NW waves per workgroup, RB blocks of 32 query rows per wave,
-// NST LDS stages per tensor.  Every wave runs ONE instruction stream per key
-// tile; tiles are issued NST-1 iterations before their first use; one
-// workgroup barrier per tile.  With RB = 2 every K/V fragment read from LDS
-// feeds two matrix instructions, and the wave needs the whole 512-entry
-// register file of its SIMD (one wave per SIMD).
+// The kernel.  NW waves per workgroup, 32 query rows per wave, NST LDS stages
+// per tensor.  Every wave runs ONE instruction stream per key tile; tiles are
+// issued NST-1 iterations before their first use; one workgroup barrier per
+// tile.  Two waves per SIMD (at most 256 registers each).
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>
-__global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(const FaKernelArgs a)
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false>
+__global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArgs a)
 {
-    constexpr int WR = 32 * RB;                   // query rows per wave
+    constexpr int WR = 32;                        // query rows per wave
     constexpr int BR = WR * NW;                   // query rows per workgroup
     constexpr int CPR = D / 8;
     constexpr int ROWB = D * 2;
@@ -448,8 +404,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     constexpr int DB = D / 32;
     constexpr int NPV = 4 * DB;                   // V^T fragments per tile: (16-key slice, head-dim block)
     constexpr int NQK = 2 * KS;                   // K fragments per tile: (head-dim slice, 32-key block)
-    constexpr int NF = NPV + NQK;                 // every fragment feeds RB matrix instructions
-    constexpr int PD = RB == 1 ? 6 : 3;           // LDS reads run this many fragments ahead
+    constexpr int NF = NPV + NQK;                 // every fragment feeds one matrix instruction
+    constexpr int PD = 6;                         // LDS reads run this many fragments ahead
     constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
     // (the first-rows path works in LDS behind the K stages that the requests for the next item fill)
     static_assert(GENERAL || LA * TILEB + NW * 32 * ROWB <= 2 * NST * TILEB, "the epilogue's row blocks do not fit behind the requested stages");
@@ -526,24 +482,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // The next work item is taken before the epilogue of the current one, and (contiguous layout) its Q^T
     // fragments and first K tiles are requested there: the 3-5 us their first bytes take to arrive from HBM lie
     // behind the epilogue instead of in front of the next tile loop.
-    u32x4 qf[RB][KS];
+    u32x4 qf[KS];
     bool next_requested = false;
     int item = take_item(0, kNoTicket);
     for (int pass = 0; item >= 0; ++pass) {
-#ifdef FA_TIMELINE
-    // (the words are collected in LDS behind the queue slot and copied out at the end of the item, so that no
-    // pointer stays live in registers across the tile loop)
-    volatile __attribute__((address_space(3))) long long *tl_lds =
-        (volatile __attribute__((address_space(3))) long long *)(uintptr_t)(lds0 + 2 * NST * TILEB + 64);
-    const long long tl_item = item;
-    if (tid == 0) {
-        unsigned hw, xc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xc));
-        tl_lds[0] = item; tl_lds[1] = ((long long)(xc & 15u) << 32) | hw; tl_lds[7] = 0; tl_lds[8] = 0;
-    }
-#endif
-    FA_TL(2);
     int bh, qblock;
     // (GENERAL with key splits: consecutive list positions are the splits of one (head, query block))
     const int n_splits = GENERAL ? a.n_splits : 1;
@@ -605,21 +547,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 
     const int q0 = qblock * BR;
     const int qw = q0 + wave * WR;          // first query row of this wave
-    const int my_q = qw + l32;              // query row of row block 0 on this lane; block b adds 32*b
+    const int my_q = qw + l32;              // query row on this lane
     const int n_rows = pack * S;            // rows of this (head | packed group)
     const bool wave_live = qw < n_rows;     // (not GENERAL: S is a multiple of 128, a live wave has all its rows)
-    // Row block b of this lane: the query position inside its head, the head relative to `bh`, whether the row
-    // exists (a row that does not exist computes on a copy of the last row and stores nothing).
-    int row_pos[RB], row_head[RB];
-    bool row_ok[RB];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-        const int r = my_q + 32 * b;
-        row_ok[b] = !GENERAL || r < n_rows;
-        const int rc = row_ok[b] ? r : n_rows - 1;
-        row_head[b] = pack > 1 ? rc / S : 0;
-        row_pos[b] = pack > 1 ? rc - row_head[b] * S : rc;
-    }
+    // This lane's row: the query position inside its head, the head relative to `bh`, whether the row exists (a
+    // row that does not exist computes on a copy of the last row and stores nothing).
+    const bool row_ok = !GENERAL || my_q < n_rows;
+    const int row_clamped = row_ok ? my_q : n_rows - 1;
+    const int row_head = pack > 1 ? row_clamped / S : 0;
+    const int row_pos = pack > 1 ? row_clamped - row_head * S : row_clamped;
     // the query positions this wave covers, for tile ranges and tile classes: its 32 rows when they lie in one
     // head, every position when they wrap from one head of a packed group into the next
     int wave_pos0 = qw, wave_npos = WR, block_pos0 = q0;
@@ -634,18 +570,12 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // Q^T fragments: B operand, lane = (query l32, head-dim slice 8*half..+7 of each 16)
     if (!next_requested) {
 #pragma unroll
-        for (int b = 0; b < RB; ++b)
-#pragma unroll
-            for (int s = 0; s < KS; ++s)
-                qf[b][s] = wave_live ? *reinterpret_cast<const u32x4 *>(
-                                           Qh + (GENERAL ? (size_t)row_head[b] * a.q_hs : 0) + (size_t)row_pos[b] * q_rs + 16 * s + 8 * half)
-                                     : u32x4{0, 0, 0, 0};
+        for (int s = 0; s < KS; ++s)
+            qf[s] = wave_live ? *reinterpret_cast<const u32x4 *>(
+                                    Qh + (GENERAL ? (size_t)row_head * a.q_hs : 0) + (size_t)row_pos * q_rs + 16 * s + 8 * half)
+                              : u32x4{0, 0, 0, 0};
     }
 
-#ifdef FA_TIMELINE      /* word 15: the wall clock when this wave's Q fragments have landed */
-    wait_vm<0>();
-    if (tid == 0) tl_lds[15] = (long long)__builtin_amdgcn_s_memrealtime();
-#endif
     const int rows_in_block = pack > 1 ? S : S - q0 < BR ? S - q0 : BR;
     int t0, t1;                 // key tiles visited by the workgroup
     fa_tile_range(Sk, kBlockKeys, a.L, a.R, block_pos0 + pos_off, rows_in_block, &t0, &t1);
@@ -715,18 +645,15 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         return cls;
     };
 
-    f32x16 o[RB][DB];
+    f32x16 o[DB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[b][db][r] = 0.0f;
-    float m_run[RB], l_a[RB], l_b[RB];      // reference point of the exponentials (raw score units), row-sum halves
-#pragma unroll
-    // (the reference point starts from a finite value far below every score: the first finite row maximum moves
-    // it, with a factor exp2(-huge) = 0 for the empty accumulators, and no place needs a test for -inf)
-    for (int b = 0; b < RB; ++b) { m_run[b] = kNoReference; l_a[b] = 0.0f; l_b[b] = 0.0f; }
+        for (int r = 0; r < 16; ++r) o[db][r] = 0.0f;
+    // reference point of the exponentials (raw score units), row-sum halves.  (The reference point starts from a
+    // finite value far below every score: the first finite row maximum moves it, with a factor exp2(-huge) = 0
+    // for the empty accumulators, and no place needs a test for -inf.)
+    float m_run = kNoReference, l_a = 0.0f, l_b = 0.0f;
     // The tile scores stay raw dot products and the softmax scale is folded into the exponent (exp2(s*c - m*c)).
     // ALiBi (mask.h:21-26 subtracts slope*|i-j| from the scaled score) enters through the matrix instruction's
     // accumulator: the first product of a key block starts from -(slope/scale)*|i-j| instead of from zero, two
@@ -736,11 +663,11 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     const float c = a.scale_log2e;
     const float cs = c;
     // (one slope per head: per lane when the rows of a wave belong to several heads of a packed group)
-    const float slope = ALIBI ? a.alibi[bh % a.H + (GENERAL ? row_head[0] : 0)] : 0.0f;
+    const float slope = ALIBI ? a.alibi[bh % a.H + (GENERAL ? row_head : 0)] : 0.0f;
     const float neg_slope_raw = ALIBI ? -slope / a.scale : 0.0f;        // per key of distance, in raw score units
     const float thresh = kRescaleLog2 / cs;
-    uint32_t pk[RB][16];        // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
-    f32x16 sx[RB][2];           // S^T of the tile whose softmax comes next: [key block 0 / 1]
+    uint32_t pk[16];            // P of the tile whose PV comes next: [0..7] keys 0..31, [8..15] keys 32..63
+    f32x16 sx[2];               // S^T of the tile whose softmax comes next: [key block 0 / 1]
 
     auto read_v = [&](uint32_t vs, int n) __attribute__((always_inline)) {
         const int t2 = n / DB, db = n % DB;
@@ -753,24 +680,21 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     };
     auto apply_mask = [&](int tile) __attribute__((always_inline)) {
         const int kb0 = tile * kBlockKeys + 4 * half;
+        const int q = row_pos + pos_off;
+        // last visible key of this query (GENERAL: the sequence may end inside the tile)
+        const int j_hi = (GENERAL && q + a.R > Sk - 1) ? Sk - 1 : q + a.R;
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            const int q = row_pos[b] + pos_off;
-            // last visible key of this query (GENERAL: the sequence may end inside the tile)
-            const int j_hi = (GENERAL && q + a.R > Sk - 1) ? Sk - 1 : q + a.R;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
-                const int j1 = j0 + 32;
-                if (j0 > j_hi || j0 < q - a.L) sx[b][0][r] = -INFINITY;
-                if (j1 > j_hi || j1 < q - a.L) sx[b][1][r] = -INFINITY;
-            }
+        for (int r = 0; r < 16; ++r) {
+            const int j0 = kb0 + 8 * (r >> 2) + (r & 3);
+            const int j1 = j0 + 32;
+            if (j0 > j_hi || j0 < q - a.L) sx[0][r] = -INFINITY;
+            if (j1 > j_hi || j1 < q - a.L) sx[1][r] = -INFINITY;
         }
     };
-    // the initial accumulator of key block `blk` of `tile` for row block b
-    auto alibi_start = [&](int b, int blk, int tile) __attribute__((always_inline)) {
+    // the initial accumulator of key block `blk` of `tile`
+    auto alibi_start = [&](int blk, int tile) __attribute__((always_inline)) {
         // signed distance of this lane's query to the lane's first key of the block: exact in fp32
-        const float base = (float)(row_pos[b] + pos_off - (tile * kBlockKeys + 32 * blk + 4 * half));
+        const float base = (float)(row_pos + pos_off - (tile * kBlockKeys + 32 * blk + 4 * half));
         f32x16 v;
         if (MASKED && a.R == 0) {
             // no visible key lies behind its query: the distance is base - k without the absolute value (the
@@ -784,50 +708,35 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         }
         return v;
     };
-    auto row_max = [&](int b) __attribute__((always_inline)) {
-        float mx = max_plain(sx[b][0][0], sx[b][1][0]);
+    auto row_max = [&]() __attribute__((always_inline)) {
+        float mx = max_plain(sx[0][0], sx[1][0]);
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, sx[b][0][r]), sx[b][1][r]);
+        for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, sx[0][r]), sx[1][r]);
         return max_of_halves(mx);
     };
-    // the decision to move the reference point of row block b; returns the factor by which everything
-    // accumulated so far has to be multiplied (1 when the reference point stays)
-    auto new_reference = [&](int b, float mx, bool &moved) __attribute__((always_inline)) {
+    // the decision to move the reference point; returns the factor by which everything accumulated so far has to
+    // be multiplied (1 when the reference point stays)
+    auto new_reference = [&](float mx, bool &moved) __attribute__((always_inline)) {
         float alpha = 1.0f;
-        const bool grow = mx > m_run[b] + thresh;   // (from kNoReference every finite maximum grows)
+        const bool grow = mx > m_run + thresh;      // (from kNoReference every finite maximum grows)
         moved = __builtin_amdgcn_ballot_w64(grow) != 0;
         if (moved) {
-            const float m_new = grow ? mx : m_run[b];
-            alpha = __builtin_amdgcn_exp2f((m_run[b] - m_new) * cs);
-            l_a[b] *= alpha;
-            l_b[b] *= alpha;
-            m_run[b] = m_new;
+            const float m_new = grow ? mx : m_run;
+            alpha = __builtin_amdgcn_exp2f((m_run - m_new) * cs);
+            l_a *= alpha;
+            l_b *= alpha;
+            m_run = m_new;
         }
         return alpha;
     };
-    auto scale_o = [&](int b, float alpha) __attribute__((always_inline)) {
+    auto scale_o = [&](float alpha) __attribute__((always_inline)) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            if (RB == 2) {
-                // O^T lives in accumulation registers, the vector ALU cannot read those: copy out, scale, copy
-                // back.  The empty statements tie every copy to this (rare) branch; without them the compiler
-                // moves the copies in front of the branch, into every iteration.
-                asm volatile("" : "+a"(o[b][db]));
-                f32x16 t = o[b][db];
-                asm volatile("" : "+v"(t));
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) t[r] *= alpha;
-                asm volatile("" : "+v"(t));
-                o[b][db] = t;
-                asm volatile("" : "+a"(o[b][db]));
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o[b][db][r] *= alpha;
-            }
-        }
+            for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
     };
-    auto p_operand = [&](int b, int t2) __attribute__((always_inline)) {
-        return u32x4{pk[b][4 * t2], pk[b][4 * t2 + 1], pk[b][4 * t2 + 2], pk[b][4 * t2 + 3]};
+    auto p_operand = [&](int t2) __attribute__((always_inline)) {
+        return u32x4{pk[4 * t2], pk[4 * t2 + 1], pk[4 * t2 + 2], pk[4 * t2 + 3]};
     };
 
     // ---- plain (not interleaved) pieces, used while the pipeline fills and drains
@@ -843,14 +752,9 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         for (int n = 0; n < NPV; ++n) {
             if (n + 2 < NPV) fr[n + 2] = read_v(vs, n + 2);
             const int t2 = n / DB, db = n % DB;
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                if (RB == 2) PinnedMfma<BF16>::pv(o[b][db], fr[n], p_operand(b, t2));
-                else o[b][db] = N::mfma(fr[n], p_operand(b, t2), o[b][db]);
-            }
+            o[db] = N::mfma(fr[n], p_operand(t2), o[db]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (RB == 2) mfma_result_wait();       // the epilogue may follow
     };
     auto qk_plain = [&](int kstage, int tile) __attribute__((always_inline)) {
         const uint32_t ks = kstage * TILEB;
@@ -858,61 +762,45 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         fr[0] = read_k(ks, 0);
         fr[1] = read_k(ks, 1);
 #pragma unroll
-        for (int b = 0; b < RB; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) { sx[b][0][r] = 0.0f; sx[b][1][r] = 0.0f; }
-        if (ALIBI) {
-#pragma unroll
-            for (int b = 0; b < RB; ++b) { sx[b][0] = alibi_start(b, 0, tile); sx[b][1] = alibi_start(b, 1, tile); }
-        }
+        for (int r = 0; r < 16; ++r) { sx[0][r] = 0.0f; sx[1][r] = 0.0f; }
+        if (ALIBI) { sx[0] = alibi_start(0, tile); sx[1] = alibi_start(1, tile); }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < NQK; ++n) {
             if (n + 2 < NQK) fr[n + 2] = read_k(ks, n + 2);
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                if (RB == 2) PinnedMfma<BF16>::qk_next(sx[b][n & 1], fr[n], qf[b][n >> 1]);
-                else sx[b][n & 1] = N::mfma(fr[n], qf[b][n >> 1], sx[b][n & 1]);
-            }
+            sx[n & 1] = N::mfma(fr[n], qf[n >> 1], sx[n & 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (RB == 2) mfma_result_wait();
     };
-    // dropout decisions of the tile whose exponentials come next: per row block and key block the sixteen
-    // bytes for this lane's sixteen keys
-    DropWords dw[RB][2];
+    // dropout decisions of the tile whose exponentials come next: per key block the sixteen bytes for this
+    // lane's sixteen keys
+    DropWords dw[2];
     auto draw_dropout = [&](int tile) __attribute__((always_inline)) {
 #pragma unroll
-        for (int b = 0; b < RB; ++b)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-                dw[b][kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)(bh + (GENERAL ? row_head[b] : 0)),
-                                          (uint32_t)(row_pos[b] + pos_off),
-                                          (uint32_t)(2 * (2 * tile + kb) + half));
+        for (int kb = 0; kb < 2; ++kb)
+            dw[kb] = dropout_words(a.seed_lo, a.seed_hi, (uint32_t)(bh + (GENERAL ? row_head : 0)),
+                                   (uint32_t)(row_pos + pos_off), (uint32_t)(2 * (2 * tile + kb) + half));
     };
-    auto dropped = [&](float e, int b, int kb, int r) __attribute__((always_inline)) {
+    auto dropped = [&](float e, int kb, int r) __attribute__((always_inline)) {
         if (!DROPOUT) return e;
-        return dropout_keep_byte(dw[b][kb], r, a.drop_threshold) ? e * a.drop_scale : 0.0f;
+        return dropout_keep_byte(dw[kb], r, a.drop_threshold) ? e * a.drop_scale : 0.0f;
     };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
         if (DROPOUT) draw_dropout(tile);
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
+        bool moved;
+        const float alpha = new_reference(row_max(), moved);
+        if (moved) scale_o(alpha);
+        const float mc = m_run * cs;
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            bool moved;
-            const float alpha = new_reference(b, row_max(b), moved);
-            if (moved) scale_o(b, alpha);
-            const float mc = m_run[b] * cs;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i], cs, -mc));
-                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][0][2 * i + 1], cs, -mc));
-                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i], cs, -mc));
-                const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[b][1][2 * i + 1], cs, -mc));
-                l_a[b] += e0; l_b[b] += e1; l_a[b] += e2; l_b[b] += e3;
-                pk[b][i] = N::pack2(dropped(e0, b, 0, 2 * i), dropped(e1, b, 0, 2 * i + 1));
-                pk[b][8 + i] = N::pack2(dropped(e2, b, 1, 2 * i), dropped(e3, b, 1, 2 * i + 1));
-            }
+        for (int i = 0; i < 8; ++i) {
+            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[0][2 * i], cs, -mc));
+            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[0][2 * i + 1], cs, -mc));
+            const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[1][2 * i], cs, -mc));
+            const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[1][2 * i + 1], cs, -mc));
+            l_a += e0; l_b += e1; l_a += e2; l_b += e3;
+            pk[i] = N::pack2(dropped(e0, 0, 2 * i), dropped(e1, 0, 2 * i + 1));
+            pk[8 + i] = N::pack2(dropped(e2, 1, 2 * i), dropped(e3, 1, 2 * i + 1));
         }
     };
 
@@ -930,67 +818,50 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         if (DROPOUT) draw_dropout(tile);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
-        bool moved[RB];
-        float alpha[RB], nmc[RB];
-#pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            alpha[b] = new_reference(b, row_max(b), moved[b]);
-            nmc[b] = -m_run[b] * cs;
-        }
-        uint32_t pn[RB][16];                       // P(tile), becomes pk at the end
-        f32x16 nx[RB][2];                          // S^T(tile+1)
+        bool moved;
+        const float alpha = new_reference(row_max(), moved);
+        float nmc = -m_run * cs;
+        uint32_t pn[16];                           // P(tile), becomes pk at the end
+        f32x16 nx[2];                              // S^T(tile+1)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < NF; ++g) {
             if (g + PD < NF) fetch(g + PD);
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                if (g < NPV) {
-                    const int t2 = g / DB, db = g % DB;
-                    if (RB == 2) PinnedMfma<BF16>::pv(o[b][db], fr[g], p_operand(b, t2));
-                    else o[b][db] = N::mfma(fr[g], p_operand(b, t2), o[b][db]);
-                } else {
-                    const int n = g - NPV;
-                    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    if (RB == 2 && n < 2) PinnedMfma<BF16>::qk_first(nx[b][n & 1], fr[g], qf[b][n >> 1]);
-                    else if (RB == 2) PinnedMfma<BF16>::qk_next(nx[b][n & 1], fr[g], qf[b][n >> 1]);
-                    else nx[b][n & 1] = N::mfma(fr[g], qf[b][n >> 1], n >= 2 ? nx[b][n & 1] : ALIBI ? alibi_start(b, n & 1, tile + 1) : zero);
-                }
-                // softmax work riding along: the 16*RB element pairs of this tile spread over the NF*RB matrix
-                // instructions, row block 0 first (its registers are free again when S^T(tile+1) is born)
-                constexpr int PAIRS = 16 * RB, SLOTS = NF * RB;
-                const int slot = g * RB + b;
-                const int p_begin = (slot * PAIRS) / SLOTS, p_end = ((slot + 1) * PAIRS) / SLOTS;
-#pragma unroll
-                for (int pi = p_begin; pi < p_end; ++pi) {
-                    // pair e of row block pb: elements (2e, 2e+1) of key block 0 for e < 8, of key block 1 for
-                    // e >= 8.  The two empty asm statements pin the arithmetic between the surrounding matrix
-                    // instructions (without them the compiler sinks all of it to the end of the iteration);
-                    // the first goes through the subtrahend, which stays in one register, so it costs no move.
-                    const int pb = pi / 16, e = pi % 16;
-                    const float x0 = e < 8 ? sx[pb][0][2 * e] : sx[pb][1][2 * (e - 8)];
-                    const float x1 = e < 8 ? sx[pb][0][2 * e + 1] : sx[pb][1][2 * (e - 8) + 1];
-                    asm volatile("" : "+v"(nmc[pb]));
-                    const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, nmc[pb]));
-                    const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, nmc[pb]));
-                    l_a[pb] += e0;
-                    l_b[pb] += e1;
-                    uint32_t packed = N::pack2(dropped(e0, pb, e >> 3, 2 * (e & 7)), dropped(e1, pb, e >> 3, 2 * (e & 7) + 1));
-                    asm volatile("" : "+v"(packed), "+v"(l_a[pb]), "+v"(l_b[pb]));
-                    pn[pb][e] = packed;
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            if (g < NPV) {
+                const int t2 = g / DB, db = g % DB;
+                o[db] = N::mfma(fr[g], p_operand(t2), o[db]);
+            } else {
+                const int n = g - NPV;
+                const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                nx[n & 1] = N::mfma(fr[g], qf[n >> 1], n >= 2 ? nx[n & 1] : ALIBI ? alibi_start(n & 1, tile + 1) : zero);
             }
-        }
-        if (RB == 2) mfma_result_wait();           // S^T(tile+1) is read by vector instructions next
+            // softmax work riding along: the 16 element pairs of this tile spread over the NF matrix instructions
+            constexpr int PAIRS = 16;
+            const int p_begin = (g * PAIRS) / NF, p_end = ((g + 1) * PAIRS) / NF;
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            if (moved[b]) scale_o(b, alpha[b]);    // rare; PV(tile-1) has been issued in full by now
-#pragma unroll
-            for (int i = 0; i < 16; ++i) pk[b][i] = pn[b][i];
-            sx[b][0] = nx[b][0];
-            sx[b][1] = nx[b][1];
+            for (int e = p_begin; e < p_end; ++e) {
+                // pair e: elements (2e, 2e+1) of key block 0 for e < 8, of key block 1 for e >= 8.  The two empty
+                // asm statements pin the arithmetic between the surrounding matrix instructions (without them the
+                // compiler sinks all of it to the end of the iteration); the first goes through the subtrahend,
+                // which stays in one register, so it costs no move.
+                const float x0 = e < 8 ? sx[0][2 * e] : sx[1][2 * (e - 8)];
+                const float x1 = e < 8 ? sx[0][2 * e + 1] : sx[1][2 * (e - 8) + 1];
+                asm volatile("" : "+v"(nmc));
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c, nmc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c, nmc));
+                l_a += e0;
+                l_b += e1;
+                uint32_t packed = N::pack2(dropped(e0, e >> 3, 2 * (e & 7)), dropped(e1, e >> 3, 2 * (e & 7) + 1));
+                asm volatile("" : "+v"(packed), "+v"(l_a), "+v"(l_b));
+                pn[e] = packed;
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        if (moved) scale_o(alpha);                 // rare; PV(tile-1) has been issued in full by now
+#pragma unroll
+        for (int i = 0; i < 16; ++i) pk[i] = pn[i];
+        sx[0] = nx[0];
+        sx[1] = nx[1];
     };
 
     unsigned ticket_ahead = kNoTicket;      // thread 0 only
@@ -1008,16 +879,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // Q has landed too (vmcnt is 0).  Touching the fragments here lets the compiler see that, so that it places
     // no vmcnt wait of its own inside the loop, where it would also wait for the asynchronous tile loads.
 #pragma unroll
-    for (int b = 0; b < RB; ++b)
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            // (64 rows per wave: from here on the fragments live in accumulation registers, where the pinned
-            // matrix instructions read them; in ordinary registers each use would cost four copies)
-            if (RB == 2) asm volatile("" : "+a"(qf[b][s]));
-            else asm volatile("" : "+v"(qf[b][s]));
-        }
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
     phase_barrier();
-    FA_TL(3);
 
     // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST
     // of its tensor, so the iteration reads K stage j % NST and V stage (j - 2) % NST; it issues the loads of
@@ -1064,9 +927,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     for (; i < t1; ++i) {                 // fill: until NST consecutive iterations are steady and the stage is 0
         if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
         generic_iteration(i, j3);
-#ifdef FA_TIMELINE
-        if (tid == 0) tl_lds[7] = tl_lds[7] + 1;
-#endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
     for (; i >= my_lo + 1 && i + NST - 1 <= my_hi - 1 && i <= t1 + 1; i += NST) {
@@ -1074,9 +934,6 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         steady_iteration(IntC<1>{}, i + 1);
         if (NST >= 3) steady_iteration(IntC<2 % NST>{}, i + 2);
         if (NST >= 4) steady_iteration(IntC<3 % NST>{}, i + 3);
-#ifdef FA_TIMELINE
-        if (tid == 0) tl_lds[8] = tl_lds[8] + NST;
-#endif
     }
     for (; i < t1; ++i) {                 // drain, up to the last two iterations
         generic_iteration(i, j3);
@@ -1088,14 +945,10 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     if (a.queue != nullptr && tid == 0) ticket_ahead = atomicAdd(&a.queue[xcd], 1u);
     for (; i <= t1 + 1; ++i) {            // the last two iterations (three stages: they request nothing any more)
         generic_iteration(i, j3);
-#ifdef FA_TIMELINE
-        if (tid == 0) tl_lds[7] = tl_lds[7] + 1;
-#endif
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
     }
 
     }   // any_tile
-    FA_TL(4);
     // rows 0..31 of a causal head are written by faithful_first_rows below instead (with key splits: in the
     // split that holds their keys, the first one; the others see none of their keys and write empty partials)
     // (GENERAL: query i sits at key position i + pos_off, so the rows concerned are those with i + pos_off < 32
@@ -1117,7 +970,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
     // ---- the next work item, and the first requests for it
     const int next_item = take_item(pass + 1, ticket_ahead);
     // (the first-rows path below works in the LDS behind the K stages that are filled here)
-    if (!GENERAL && RB == 1 && next_item >= 0) {
+    if (!GENERAL && next_item >= 0) {
         int nbh, nqb, nt0, nt1;
         fa_item_decode(next_item, a.BH, a.n_qblocks, a.descending, &nbh, &nqb);
         const uint16_t *nQ, *nK, *nV;
@@ -1143,7 +996,7 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         const int nrow = nq0 + (nq0 + wave * WR < S ? wave * WR : 0) + l32;
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-            qf[0][s] = *reinterpret_cast<const u32x4 *>(nQ + (size_t)nrow * q_rs + 16 * s + 8 * half);
+            qf[s] = *reinterpret_cast<const u32x4 *>(nQ + (size_t)nrow * q_rs + 16 * s + 8 * half);
         next_requested = true;
     }
     // With key splits the item writes fp32 partial results, (O normalised over its own keys, logsumexp of its
@@ -1154,35 +1007,31 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
         o_part = a.o_part + part * S * D;
         lse_part = a.lse_part + part * S;
     }
-    if (wave_live) {
-        // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides)
-#pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            if (!GENERAL && faithful && wave == 0 && b == 0) continue;
+    // ---- epilogue: O / l, logsumexp (the reference has none; flash_forward.h:318-327 only divides).  Not for a
+    // row past the end, nor for rows that faithful_first_rows writes below.
+    const bool own_store = wave_live && row_ok && !(!GENERAL && faithful && wave == 0) && !(GENERAL && my_q < f_rows);
+    if (own_store) {
+        {
             // the row's index in its head's [S, ...] output, counted from head `bh` (packed groups: row_head
             // heads further on; their logsumexp and partial rows follow at S per head, their O rows at o_hs)
-            const int q = GENERAL ? row_head[b] * S + row_pos[b] : my_q + 32 * b;
-            if (!row_ok[b]) continue;              // a row past the end
-            if (GENERAL && b == 0 && my_q < f_rows) continue;      // written by faithful_first_rows below
-            const float l_half = l_a[b] + l_b[b];
+            const int q = GENERAL ? row_head * S + row_pos : my_q;
+            const float l_half = l_a + l_b;
             const float l_tot = l_half + swap_halves(l_half);
             const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
             const float inv = empty ? 0.0f : 1.0f / l_tot;
             const float lse_row = empty ? -INFINITY
-                                        : m_run[b] * a.scale + __builtin_logf(l_tot);
+                                        : m_run * a.scale + __builtin_logf(l_tot);
             if (GENERAL && o_part != nullptr) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        const f32x4 w = {o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv, o[b][db][4 * g + 2] * inv,
-                                         o[b][db][4 * g + 3] * inv};
+                        const f32x4 w = {o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv,
+                                         o[db][4 * g + 3] * inv};
                         *reinterpret_cast<f32x4 *>(o_part + (size_t)q * D + 32 * db + 8 * g + 4 * half) = w;
                     }
                 if (half == 0) lse_part[q] = lse_row;
-                continue;
-            }
-            if (!GENERAL && RB == 1) {
+            } else if (!GENERAL) {
                 // Through LDS, so that every store instruction writes whole rows: a lane holds 8-byte pieces of ONE
                 // row, and stored from the registers an instruction touches 32 rows with 16 bytes each (the
                 // address path takes as long for it as for 32 full cache lines); row-major, four (eight) rows of
@@ -1202,8 +1051,8 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
                         u32x2 w;
-                        w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
-                        w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
+                        w[0] = N::pack2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv);
+                        w[1] = N::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
                         const int chunk = 4 * db + g;           // 16-byte chunk of the row: elements 8 * chunk .. + 7
                         *(lds_u32x2 *)(uintptr_t)(obase + l32_e * ROWB + ((chunk ^ (l32_e & (CPR - 1))) << 4) + 8 * half_e) = w;
                     }
@@ -1222,29 +1071,20 @@ __global__ void __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) fa_fwd_pipelined(con
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     u32x2 w;
-                    w[0] = N::pack2(o[b][db][4 * g] * inv, o[b][db][4 * g + 1] * inv);
-                    w[1] = N::pack2(o[b][db][4 * g + 2] * inv, o[b][db][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2 *>(Oh + (GENERAL ? (size_t)row_head[b] * a.o_hs + (size_t)row_pos[b] * o_rs : (size_t)q * o_rs) +
+                    w[0] = N::pack2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv);
+                    w[1] = N::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2 *>(Oh + (GENERAL ? (size_t)row_head * a.o_hs + (size_t)row_pos * o_rs : (size_t)q * o_rs) +
                                                32 * db + 8 * g + 4 * half) = w;
                 }
             }
-            if (a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
+            if (!(GENERAL && o_part != nullptr) && a.lse != nullptr && half == 0) a.lse[(size_t)bh * S + q] = lse_row;
         }
     }
-    FA_TL(5);
     if (!GENERAL && fr1 > fr0) __syncthreads();       // (the epilogue's LDS blocks have been read by their waves)
     if (fr1 > fr0)    // the LDS behind the first LA K stages is free
         faithful_first_rows<BF16, D>(Qh, Kh, Vh, Oh, o_part, o_part != nullptr ? lse_part : a.lse != nullptr ? a.lse + (size_t)bh * S : nullptr,
                                      fr0, fr1, pos_off, a.L, a.scale, slope, q_rs, k_rs, v_rs, o_rs, DROPOUT ? a.drop_threshold : 0u, a.drop_scale,
                                      a.seed_lo, a.seed_hi, (uint32_t)bh, lds0 + LA * TILEB);
-    FA_TL(6);
-#ifdef FA_TIMELINE
-    if (tid == 0 && g_fa_timeline != nullptr) {
-        tl_lds[9] = ((long long)t0 << 32) | (unsigned)t1;
-        for (int w = 0; w < 16; ++w) g_fa_timeline[16 * tl_item + w] = tl_lds[w];
-    }
-    __syncthreads();
-#endif
     item = next_item;
     }   // next work item
     // the last workgroup to leave rewinds the queue for the next launch that uses it
@@ -1293,16 +1133,12 @@ __global__ void __launch_bounds__(256) fa_combine_splits(const FaKernelArgs a)
     if (a.lse != nullptr && c4 == 0) a.lse[row] = mx == -INFINITY ? -INFINITY : mx + __logf(wsum);
 }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int RB, int NST, bool STRIDED = false>
-hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false>
+hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream, bool configure_only)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
-#ifdef FA_TIMELINE
-    const size_t smem = 2 * NST * TILEB + 64 + 128;
-#else
     const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the two words of the queue schedule
-#endif
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, RB, NST, STRIDED>;
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, NST, STRIDED>;
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
     const unsigned long long dev_bit = 1ull << fa_launch_device();
@@ -1311,6 +1147,7 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
         if (e != hipSuccess) return e;
         configured.fetch_or(dev_bit, std::memory_order_relaxed);
     }
+    if (configure_only) return hipSuccess;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, a);
     return hipGetLastError();
 }
@@ -1318,42 +1155,44 @@ hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream)
 
 // shape 0: 8 waves x 32 rows = 256 query rows per workgroup, three LDS stages, one workgroup per CU.
 // shape 1: 4 waves x 32 rows = 128 query rows per workgroup, two LDS stages, two workgroups per CU.
-// (RB = 2, 64 rows per wave with one wave per SIMD, compiles but is not instantiated: the register allocator
-// answers it with about 500 AGPR<->VGPR moves per tile.)
 // (The 8-wave general instantiations get two LDS stages instead of three: a third buys nothing measurable --
 // c3's shape stored [B,S,H,D] runs at 925 TFLOP/s with two and 929 with three, c2's at 553 against 514 -- and
 // two leave LDS for a second workgroup of the small shapes.)
-#ifndef FA_NST8
-#define FA_NST8 3
-#endif
-#ifndef FA_NST8_GENERAL
-#define FA_NST8_GENERAL 2
-#endif
-#ifndef FA_ROWS64       /* 1: the 64-rows-per-wave shape for head dimension 128, contiguous layout (under evaluation) */
-#define FA_ROWS64 0
-#endif
-#if FA_ROWS64
-#define FA_ROWS64_CASE(BF, DD, MK, AL) \
-    if (shape == 0 && !GENERAL && DD == 128 && !AL) return launch<BF != 0, DD, MK != 0, false, false, false, 4, 2, 3>(a, grid, stream);
-#else
-#define FA_ROWS64_CASE(BF, DD, MK, AL)
-#endif
 template <bool GENERAL, bool DROPOUT, bool STRIDED = false>
-hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream)
+hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid, hipStream_t stream,
+                          bool configure_only = false)
 {
     const int alibi = a.alibi != nullptr;
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
-        FA_ROWS64_CASE(BF, DD, MK, AL) \
-        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, 1, (GENERAL ? FA_NST8_GENERAL : FA_NST8), STRIDED>(a, grid, stream); \
-        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 1, 2, STRIDED>(a, grid, stream); \
+        if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, (GENERAL ? 2 : 3), STRIDED>(a, grid, stream, configure_only); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 2, STRIDED>(a, grid, stream, configure_only); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
     FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)
 #undef FA_CASES
 #undef FA_CASE
-#undef FA_ROWS64_CASE
     return hipErrorInvalidValue;
+}
+
+// The LDS opt-in of every instantiation of one flavour, for the current device, without launching anything: what
+// fa_init() runs so that no later launch has to (hipFuncSetAttribute is not a stream operation and must not
+// fall into a stream capture).
+template <bool GENERAL, bool DROPOUT, bool STRIDED = false>
+hipError_t configure_forward()
+{
+    FaKernelArgs a = {};
+    static const float slope_stand_in = 0.0f;      // (only tested against null)
+    for (int bf16 = 0; bf16 < 2; ++bf16)
+        for (int D = 64; D <= 128; D += 64)
+            for (int masked = 0; masked < 2; ++masked)
+                for (int alibi = 0; alibi < 2; ++alibi)
+                    for (int shape = 0; shape < 2; ++shape) {
+                        a.alibi = alibi ? &slope_stand_in : nullptr;
+                        const hipError_t e = launch_forward<GENERAL, DROPOUT, STRIDED>(a, bf16, D, masked, shape, 0u, nullptr, true);
+                        if (e != hipSuccess) return e;
+                    }
+    return hipSuccess;
 }
 
 }  // namespace

@@ -13,3 +13,4 @@ hipError_t fa_launch_forward_strided(const FaKernelArgs &a, int bf16, int D, int
 {
     return launch_forward<false, false, true>(a, bf16, D, masked, shape, grid, stream);
 }
+hipError_t fa_configure_forward_strided() { return configure_forward<false, false, true>(); }

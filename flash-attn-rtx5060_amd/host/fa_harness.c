@@ -201,6 +201,11 @@ int main(int argc, char **argv)
         /* gradients of sum(dO * O) through fa_bwd, with dO from the same generator (tensor slot of Q, seed + 1000):
            a second JSON line; the forward pass above has left O and the logsumexp on the device */
         if (!c.lse) { fprintf(stderr, "--backward needs the logsumexp (drop --no-lse)\n"); return 2; }
+        /* fa_bwd recomputes P from exact scores: hand it the O and logsumexp of a forward pass whose first rows
+           use exact products too (the default recomputes a causal head's first 32 rows in the CPU verifier's
+           rounded-product arithmetic, which is what the check of the forward output above wants) */
+        p.exact_first_rows = 1;
+        if (check(fa_fwd(&p, NULL), "forward launch for the backward pass") || check(fa_dev_sync(), "sync")) return 1;
         void *dg[4] = {NULL, NULL, NULL, NULL}, *ws = NULL;
         for (int t = 0; t < 4; ++t) {
             hg[t] = malloc(bytes);

@@ -22,7 +22,14 @@ typedef struct fa_bwd_params {
     const void *Q, *K, *V;    /* device, the forward inputs: Q [B,N,S,d]; K, V [B,n_kv_heads,S_kv,d]              */
     const void *O;            /* [B,N,S,d] device, the forward output                                          */
     const void *dO;           /* [B,N,S,d] device, gradient of the loss with respect to O                      */
-    const float *L;           /* [B,N,S] contiguous fp32 logsumexp written by the forward pass                  */
+    const float *L;           /* [B,N,S] contiguous fp32 logsumexp written by the forward pass.  Run that pass
+                                 with fa_fwd_params.exact_first_rows = 1: the backward pass recomputes P from
+                                 exact scores, and the default forward writes the first 32 rows of a causal
+                                 head (rows that see at most 32 keys) in the reference verifier's
+                                 rounded-product arithmetic.  With the default forward's O and L those rows'
+                                 gradients are still within 2e-3 (fp16) / 1.6e-2 (bf16) of the largest
+                                 gradient at unit-variance inputs (tests/test_gpu_parity_bwd.py); every other
+                                 row is unaffected                                                             */
     void *dQ, *dK, *dV;       /* device, shaped like Q, K, V; fully overwritten, same type as the inputs        */
     int B, N, S, d;
     float softmax_scale;

@@ -128,9 +128,11 @@ unsigned long long fa_fwd_workspace_bytes(const fa_fwd_params *p);
 /* A split count that fills the device for these shapes (1 when the problem has enough work items anyway). */
 int fa_fwd_suggest_splits(const fa_fwd_params *p);
 
-/* Optional: sets up the library's state for the current device (looks up the addresses of its two
- * file-scope device arrays and the CU count) so that the first fa_fwd call does not.  Every entry point that
- * needs the state does the same on its first call on a device. */
+/* Sets up the library's state for the current device: looks up the addresses of its two file-scope device
+ * arrays and the CU count, and makes the LDS opt-in (hipFuncSetAttribute) of every kernel instantiation.  Optional
+ * for eager use -- every entry point does what it still needs on its first call on a device -- but CALL IT BEFORE
+ * A STREAM CAPTURE on that device: those first-call steps are not stream operations, and after fa_init() no
+ * entry point makes any HIP call other than its kernel launches, hipStreamIsCapturing and hipStreamGetId. */
 int fa_init(void);
 
 /* Enqueues the forward pass on `stream` and returns without synchronising.
@@ -156,14 +158,20 @@ unsigned long long fa_fwd_static_scratch_bytes(void);
 
 /* FA_SCHED_QUEUE keeps its counters in the library's own device memory: 256 sets per device; the last workgroup
  * of a launch rewinds its set.  Eager launches: a set belongs to a stream (launches on one stream run one after
- * the other and may share it); the first 16 streams that launch on a device get one each and keep it for the life
- * of the process, launches on further streams walk the work list with FA_SCHED_PERSISTENT's fixed order instead
- * (same results, no counters).  Every launch captured into a graph gets a set of its own, for good (a replay may
- * run next to anything): 240 per device and process, after which captured launches use the fixed order as well.
- * No two launches that can run at the same time share counters.  A launch that was killed half-way (device
- * reset, process signal) leaves its set dirty: fa_reset_work_queues() waits for the device, zeroes all sets of
- * the current device and forgets which stream owned which.  Never call it while launches are being captured. */
+ * the other and may share it), named by its handle and, where the loaded HIP runtime has hipStreamGetId (7.1 and
+ * later), its runtime id, so that a new stream that happens to get a destroyed stream's handle value does not
+ * inherit its set; with an older runtime the handle alone names it, and the release call below is required.  At most 16 streams of a device own
+ * a set at a time; a stream keeps its set until fa_release_work_queue(stream) (call it before destroying a
+ * stream that launched with the queue schedule; it waits for the stream) or fa_reset_work_queues().  Launches on
+ * further streams, and on hipStreamPerThread (one handle value for a different stream in every host thread),
+ * walk the work list with FA_SCHED_PERSISTENT's fixed order instead: same results, no counters.  Every launch
+ * captured into a graph gets a set of its own, for good (a replay may run next to anything): 240 per device and
+ * process, after which captured launches use the fixed order as well.  No two launches that can run at the same
+ * time share counters.  A launch that was killed half-way (device reset, process signal) leaves its set dirty:
+ * fa_reset_work_queues() waits for the device, zeroes all sets of the current device and forgets which stream
+ * owned which.  Never call it while launches are being captured. */
 int fa_reset_work_queues(void);
+int fa_release_work_queue(void *stream);
 
 /*
  * The reference's entry point, same name, argument order and meaning

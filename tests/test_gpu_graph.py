@@ -102,3 +102,56 @@ def test_more_captured_queue_launches_than_counter_sets(fa):
         torch.cuda.synchronize()
         for o in outs:
             assert torch.equal(o.view(torch.int16), want.view(torch.int16)), replay
+
+
+FIRST_CALL_SCRIPT = r"""
+import ctypes, sys
+sys.path.insert(0, {repo!r}); sys.path.insert(0, {tests!r})
+import torch
+from __graft_entry__ import load_package
+fa = load_package()
+L = fa.lib()
+assert L.fa_init() == fa.FA_OK
+# decoding-shaped problem with key splits through the entry point that allocates nothing, queue schedule forced:
+# the capture below is the library's FIRST launch in this process
+B, H, Hk, S, Skv, D = 2, 8, 2, 4, 2048, 128
+g = torch.Generator(device="cuda").manual_seed(3)
+q = torch.randn((B, H, S, D), device="cuda", generator=g).half()
+k, v = (torch.randn((B, Hk, Skv, D), device="cuda", generator=g).half() for _ in range(2))
+o = torch.full_like(q, float("nan"))
+lse = torch.full((B, H, S), float("nan"), dtype=torch.float32, device="cuda")
+p = fa.make_params(B, H, S, D, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), causal=True,
+                   n_kv_heads=Hk, S_kv=Skv, split_num=4, sched=3)
+torch.cuda.synchronize()
+side = torch.cuda.Stream()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+        st = L.fa_fwd_split_static(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+assert st == fa.FA_OK, st
+torch.cuda.synchronize()
+for replay in range(3):
+    for t in (q, k, v):
+        t.copy_(torch.randn(t.shape, device="cuda", generator=g).half())
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    want, want_lse = fa.flash_attention_forward(q, k, v, causal=True, splits=4, sched=3)
+    torch.cuda.synchronize()
+    assert torch.equal(o.view(torch.int16), want.view(torch.int16)) and torch.equal(lse, want_lse), replay
+print("captured first call ok")
+"""
+
+
+def test_capture_as_the_first_call_after_fa_init():
+    """fa_init() does everything that is not a stream operation (device arrays' addresses, CU count, the LDS
+    opt-in of every kernel), so a stream capture may contain the library's very first launch.  Needs a process of
+    its own: in this one the library has long been used."""
+    import os
+    import subprocess
+    import sys
+    tests = os.path.dirname(os.path.abspath(__file__))
+    repo = os.path.dirname(tests)
+    proc = subprocess.run([sys.executable, "-c", FIRST_CALL_SCRIPT.format(repo=repo, tests=tests)], stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert proc.returncode == 0 and "captured first call ok" in proc.stdout, proc.stdout[-3000:]

@@ -159,3 +159,64 @@ def test_queue_schedule_on_many_streams_at_once(fa):
     torch.cuda.synchronize()
     for o, l in outs:
         assert torch.equal(o.view(torch.int16), o_ref.view(torch.int16)) and torch.equal(l, l_ref)
+
+
+def test_queue_schedule_on_the_per_thread_stream_from_two_threads(fa):
+    """hipStreamPerThread is ONE handle value for a different stream in every host thread: two threads that launch
+    the queue schedule on it at the same time must not share a counter set (they would skip or repeat work items).
+    The library gives that handle no counters at all -- the fixed work order, same bits."""
+    import ctypes
+    import threading
+    import torch
+    shape, dtype = (2, 16, 2048, 128), 0
+    q, k, v = make_inputs(fa, shape, dtype, seed=94)
+    tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    o_ref, l_ref = fa.flash_attention_forward(tq, tk, tv, causal=True, sched=1)
+    torch.cuda.synchronize()
+    per_thread = ctypes.c_void_p(2)                 # hipStreamPerThread
+    L = fa.lib()
+    B, H, S, D = shape
+    outs, status = [], []
+
+    def worker():
+        mine = []
+        for _ in range(6):
+            o = torch.full_like(o_ref, float("nan"))
+            l = torch.full_like(l_ref, float("nan"))
+            p = fa.make_params(B, H, S, D, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(), l.data_ptr(),
+                               causal=True, dtype=dtype, sched=3)
+            status.append(L.fa_fwd(ctypes.byref(p), per_thread))
+            mine.append((o, l))
+        outs.extend(mine)
+
+    torch.cuda.synchronize()                        # (the tensors above were filled on torch's stream)
+    threads = [threading.Thread(target=worker) for _ in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert status == [fa.FA_OK] * 12
+    for o, l in outs:
+        assert torch.equal(o.view(torch.int16), o_ref.view(torch.int16)) and torch.equal(l, l_ref)
+
+
+def test_streams_that_come_and_go_release_their_counter_sets(fa):
+    """Forty streams, one after the other, each launching the queue schedule and then releasing its counter set
+    (fa_release_work_queue) before it is destroyed: more streams than a device has eager sets; every result is the
+    reference's bits, and a stream created afterwards still finds a set (observable only as a correct result)."""
+    import ctypes
+    import torch
+    shape, dtype = (1, 16, 2048, 128), 0
+    q, k, v = make_inputs(fa, shape, dtype, seed=95)
+    tq, tk, tv = (to_torch(x, dtype) for x in (q, k, v))
+    o_ref, l_ref = fa.flash_attention_forward(tq, tk, tv, causal=True, sched=1)
+    torch.cuda.synchronize()
+    for n in range(40):
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            o, l = fa.flash_attention_forward(tq, tk, tv, causal=True, sched=3)
+        assert fa.lib().fa_release_work_queue(ctypes.c_void_p(s.cuda_stream)) == fa.FA_OK      # waits for the stream
+        assert torch.equal(o.view(torch.int16), o_ref.view(torch.int16)) and torch.equal(l, l_ref), n
+        del s
+

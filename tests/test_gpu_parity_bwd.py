@@ -50,7 +50,7 @@ def test_gradients_against_the_fp64_oracle(fa, oracle, shape, dtype, causal, wl,
     do, _, _ = make_inputs(fa, shape, dtype, seed=501 + shape[2])
     dq_ref, dk_ref, dv_ref = oracle.bwd_f64(q, k, v, do, dtype, None, causal, wl, wr)
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
-    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr)
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, exact_first_rows=True)
     dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr)
     torch.cuda.synchronize()
     for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
@@ -59,13 +59,41 @@ def test_gradients_against_the_fp64_oracle(fa, oracle, shape, dtype, causal, wl,
         check(err, dtype, name)
 
 
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_default_forward_feeding_the_backward_pass(fa, oracle, dtype):
+    """fa_bwd.h asks for a forward pass with exact_first_rows = 1.  A C caller that forgets (the default forward
+    writes the first 32 rows of a causal head in the CPU verifier's rounded-product arithmetic, and fa_bwd
+    recomputes P from exact scores) must still get gradients inside the ordinary bars: stated bound, rows 0-31 of
+    dQ and all of dK, dV within rel-L2 1e-3 / 8e-3 and max-abs 2e-3 / 1.6e-2 of the largest gradient; dQ rows
+    from 32 on do not change by a bit (a row of dQ depends on its own O row and logsumexp only)."""
+    import torch
+    shape = (1, 2, 256, 128)
+    q, k, v = make_inputs(fa, shape, dtype, seed=901)
+    do, _, _ = make_inputs(fa, shape, dtype, seed=902)
+    dq_ref, dk_ref, dv_ref = oracle.bwd_f64(q, k, v, do, dtype, None, True, -1, -1)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    grads = {}
+    for exact in (False, True):
+        o, lse = fa.flash_attention_forward(tq, tk, tv, causal=True, exact_first_rows=exact)
+        grads[exact] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=True)
+    torch.cuda.synchronize()
+    for name, got, want in zip(("dQ", "dK", "dV"), grads[False], (dq_ref, dk_ref, dv_ref)):
+        err = grad_errors(oracle.to_f32(from_torch(got), dtype), want)
+        print("default forward", dtype, name, err, flush=True)
+        check(err, dtype, name)
+    first = grad_errors(oracle.to_f32(from_torch(grads[False][0][:, :, :32].contiguous()), dtype), dq_ref[:, :, :32])
+    print("default forward", dtype, "dQ rows 0-31", first, flush=True)
+    check(first, dtype, "dQ rows 0-31")
+    assert torch.equal(grads[False][0][:, :, 32:], grads[True][0][:, :, 32:])
+
+
 def test_against_torch_autograd_on_the_gpu(fa):
     """A larger problem than the CPU oracle finishes quickly: torch's fp32 attention and autograd on the GPU."""
     import torch
     B, H, S, D = 2, 4, 2048, 128
     g = torch.Generator(device="cuda").manual_seed(5)
     q, k, v, do = (torch.randn((B, H, S, D), device="cuda", generator=g).half() for _ in range(4))
-    o, lse = fa.flash_attention_forward(q, k, v, causal=True)
+    o, lse = fa.flash_attention_forward(q, k, v, causal=True, exact_first_rows=True)
     dq, dk, dv = fa.flash_attention_backward(q, k, v, o, lse, do, causal=True)
     qf, kf, vf = (t.float().requires_grad_(True) for t in (q, k, v))
     ref = torch.nn.functional.scaled_dot_product_attention(qf, kf, vf, is_causal=True)
