@@ -129,11 +129,11 @@ def backward_bench(args):
     slopes = np.power(2.0, -8.0 / H * (np.arange(H) + 1)).astype(np.float32) if args.alibi else None
     kw = dict(causal=causal, window_left=wl, dropout_prob=args.dropout, seed=48,
               alibi_slopes=torch.from_numpy(slopes).cuda() if args.alibi else None)
-    o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
+    o, lse = fa.flash_attention_forward(tq, tk, tv, exact_first_rows=True, **kw)      # the pairing fa_bwd.h asks for
     grads = [None]
 
     def step():
-        grads[0] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
+        grads[0] = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products="auto" if args.bwd_form == "five" else False, **kw)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -211,6 +211,9 @@ def main():
     ap.add_argument("--kv-heads", type=int, default=0, metavar="N",
                     help="K and V with N heads, shared by groups of query heads (not the headline metric)")
     ap.add_argument("--backward", action="store_true", help="time the backward pass on the workload's shape (not the headline metric)")
+    ap.add_argument("--bwd-form", default="five", choices=("five", "seven"),
+                    help="--backward: five = dS blocks through a B*H*S*S-element workspace and dQ as one product over them "
+                         "(reference layout only; other problems fall back to seven); seven = S and dP recomputed by both kernels")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device-to-device copy kernel of this size (for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters to bytes)")

@@ -50,7 +50,7 @@ EXPORTED_SYMBOLS = (
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_heads", "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
-    "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_algorithmic_flops",
+    "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_fast_workspace_bytes", "fa_bwd_algorithmic_flops",
     "fa_bwd_sched_query_tile_range", "fa_bwd_sched_classify",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
@@ -155,6 +155,8 @@ def lib():
         L.fa_bwd.argtypes = [ctypes.POINTER(FaBwdParams), ctypes.c_void_p]
         L.fa_bwd_workspace_bytes.restype = ctypes.c_ulonglong
         L.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd_fast_workspace_bytes.restype = ctypes.c_ulonglong
+        L.fa_bwd_fast_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
         L.fa_bwd_algorithmic_flops.restype = ctypes.c_double
         L.fa_bwd_algorithmic_flops.argtypes = [ctypes.c_int] * 7
         L.fa_bwd_sched_query_tile_range.restype = None
@@ -320,10 +322,13 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
 
 
 def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                             alibi_slopes=None, dropout_prob=0.0, seed=0):
+                             alibi_slopes=None, dropout_prob=0.0, seed=0, five_products="auto"):
     """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
     fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask, slopes, dropout
     probability and seed.
+    ``five_products``: True asks for the workspace that selects the five-product form (fa_bwd_fast_workspace_bytes:
+    B*N*S*S elements more), False for the small one; "auto" takes the large one when the problem qualifies and it
+    is at most a quarter of the device's free memory.
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
     import torch
@@ -361,12 +366,23 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
                         alibi_ptr=0 if alibi_slopes is None else alibi_slopes.data_ptr(), strides=strides,
                         dropout_prob=dropout_prob, seed=seed)
     need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
-    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    fast = lib().fa_bwd_fast_workspace_bytes(ctypes.byref(p)) if five_products else 0
+    if fast and (five_products is True or fast <= _ws_budget(q.device)):
+        need = fast
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)     # stream-ordered: freed after the launch
     p.workspace, p.workspace_bytes = workspace.data_ptr(), need
     st = lib().fa_bwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream))
     if st != FA_OK:
         raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
     return dq, dk, dv
+
+
+def _ws_budget(device):
+    """A quarter of the memory a new allocation could get: the device's free memory plus what torch's allocator
+    holds without using it."""
+    import torch
+    free, _ = torch.cuda.mem_get_info(device)
+    return (free + torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)) // 4
 
 
 _autograd_function = None

@@ -15,6 +15,12 @@ struct FaBwdArgs {
     float *delta;                           // [B,H,S] scratch: sum_t dO*O per row, written by fa_bwd_dq
     float *lse2;                            // [B,H,S] scratch: lse * log2(e), +inf for rows that saw no key
     uint16_t *dQ, *dK, *dV;
+    // Five-product form (reference layout only), or null: dS in blocks of 32 queries x 32 keys, 2 KiB each, block
+    // (head bh, query block i, key block j) at (bh * fa_ds_blocks_per_head + fa_ds_block_index(i, j)) * 2 KiB
+    // (fa_bwd_layout.h).  Inside a block the first KiB
+    // holds, for 16-byte slot 32 h + k, key k against the queries 4 h + {0..3, 8..11}; the second KiB the same for
+    // the queries 16 + 4 h + {0..3, 8..11} (h = 0, 1): the order in which fa_bwd_dkdv's lanes hold them.
+    uint16_t *ds_blocks;
     const float *alibi;                     // [H] slopes or NULL
     FaBwdTensor q, k, v, o, dO_, dq, dk, dv;
     int B, H, Hk;                           // query heads, K/V heads (Hk divides H)

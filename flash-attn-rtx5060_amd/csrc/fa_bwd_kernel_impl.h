@@ -34,6 +34,7 @@ namespace {
 constexpr int kBwdWaves = 8;            // 8 waves x 32 owned rows = 256 rows per workgroup, two waves per SIMD
 constexpr int kBwdStages = 3;           // LDS ring: with three stages one barrier per tile is enough
 constexpr float kLog2e = 1.44269504088896340736f;
+constexpr int kDsBlockBytes = 2048;     // one 32-query x 32-key block of dS in the storage type
 
 // Takes the word by value on purpose: __builtin_bit_cast applied directly to an element of a vector
 // (`__builtin_bit_cast(float, v[e])`) reads element 0 whatever e is with this compiler.
@@ -120,6 +121,30 @@ __device__ __forceinline__ void dma_4(const float *src, int index, uint32_t lds)
     const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
     const uint32_t voff = (uint32_t)index * 4u;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform run-time n (the instruction takes an immediate)
+__device__ __forceinline__ void wait_vm_upto(int n)
+{
+    switch (n) {
+#define FA_WAIT_CASE(k) case k: wait_vm<k>(); break;
+    FA_WAIT_CASE(0) FA_WAIT_CASE(1) FA_WAIT_CASE(2) FA_WAIT_CASE(3) FA_WAIT_CASE(4) FA_WAIT_CASE(5) FA_WAIT_CASE(6) FA_WAIT_CASE(7)
+    FA_WAIT_CASE(8) FA_WAIT_CASE(9) FA_WAIT_CASE(10) FA_WAIT_CASE(11) FA_WAIT_CASE(12) FA_WAIT_CASE(13) FA_WAIT_CASE(14) FA_WAIT_CASE(15)
+    FA_WAIT_CASE(16)
+#undef FA_WAIT_CASE
+    default: wait_vm<0>(); break;
+    }
+}
+
+// dma_16 with the streaming hint: data that is read exactly once should not displace what others re-read from L2
+__device__ __forceinline__ void dma_16_stream(const char *base, uint32_t voff, uint32_t lds)
+{
+    const uint64_t b = (uint64_t)base;
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint64_t ub = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                  :: "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(voff), "s"(ub) : "memory", "m0");
 }
 
@@ -356,14 +381,18 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
 // LDS stage: Q (row-wise for S = Q K^T, transposed for dK^T += Q^T dS), dO (row-wise for dP = dO V^T, transposed
 // for dV^T += dO^T P), 64 rescaled logsumexps, 64 deltas.
 // ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
+// WRITE_DS (reference layout only): every 32-query x 32-key block of dS that a wave forms is also written to
+// a.ds_blocks, in the wave's operand order, for fa_bwd_dq_from_ds.
+template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, bool WRITE_DS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
     constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
+    static_assert(!WRITE_DS || LAYOUT == 0, "dS blocks are written for the reference's layout only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
     constexpr int KS = Reader::KS, DB = Reader::DB, TILEB = Loader::TILEB, STAGEB = 2 * TILEB + 512, IPW = Loader::IPW;
+    constexpr int NSTG = kBwdStages;                                  // LDS stages; pairs are requested NSTG - 1 ahead
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
@@ -416,7 +445,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     uint32_t stat_addr = lds0 + 2 * TILEB + 16 * half;       // this lane's logsumexp / delta words in the stage being read
     // dropout: 128 bytes per wave behind the ring, through which keep bits drawn with the query on the lane (one
     // Philox block covers sixteen keys of ONE query) reach the lanes that own the keys
-    const uint32_t drop_lds = lds0 + kBwdStages * STAGEB + wave * 128;
+    const uint32_t drop_lds = lds0 + NSTG * STAGEB + wave * 128;
     Loader ldq, ldg;
     if (!STRIDES || GENERAL) ldq.init(wave, lane, q_rs * 2);      // (general: only its ragged tiles go through these two)
     if (GENERAL) ldg.init(wave, lane, g_rs * 2);
@@ -475,6 +504,18 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     f32x16 dk[DB], dv[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) { dk[db] = zero16(); dv[db] = zero16(); }
+    // WRITE_DS, head dimension 128: the kernel needs every register it can have (two waves per SIMD: 256), and a
+    // value the compiler spills to scratch memory inside the tile loop comes back behind a wait for ALL loads and
+    // stores in flight.  The last PARKED of the K^T and V^T fragments, which every half tile uses once, are kept in
+    // LDS instead (32 bytes per lane and fragment pair, written once per work item) and read like any A operand.
+    constexpr int PARKED = WRITE_DS && D == 128 ? 1 : 0;
+    const uint32_t park_lds = lds0 + NSTG * STAGEB;
+    auto parked = [&](int which, int s) __attribute__((always_inline)) {
+        uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(ln));
+        const uint32_t addr = park_lds + 32u * PARKED * ((uint32_t)wave * 64u + ln) + 32u * (uint32_t)(s - (KS - PARKED)) + 16u * which;
+        return *(volatile __attribute__((address_space(3))) u32x4 *)(uintptr_t)addr;
+    };
 
     // 32 queries (block qb of the tile in the stage being read) against this wave's 32 keys
     auto half_tile = [&](bool edge, float slope_l2, uint32_t bhq, int t, int qb) __attribute__((always_inline)) {
@@ -490,7 +531,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
         }
         f32x16 sx = zero16();            // rows = queries, column (lane) = key
 #pragma unroll
-        for (int s = 0; s < KS; ++s) sx = N::mfma(rd.rows(q_tile, s, qb), kf[s], sx);      // S = Q K^T
+        for (int s = 0; s < KS; ++s) sx = N::mfma(rd.rows(q_tile, s, qb), s >= KS - PARKED ? parked(0, s) : kf[s], sx);      // S = Q K^T
         const int first = t * 64 + 32 * qb + 4 * half;                      // query of accumulator row 0 on this lane
         if (MASKED && edge) {            // wave-uniform; a masked score becomes -inf and its P exactly 0
             int hi = my_k + Rq, lo = my_k - Lq - first;                      // visible: lo <= 8*(r/4) + r%4 <= hi
@@ -540,7 +581,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
         }
         f32x16 dp = zero16();
 #pragma unroll
-        for (int s = 0; s < KS; ++s) dp = N::mfma(rd.rows(g_tile, s, qb), vf[s], dp);      // dP = dO V^T
+        for (int s = 0; s < KS; ++s) dp = N::mfma(rd.rows(g_tile, s, qb), s >= KS - PARKED ? parked(1, s) : vf[s], dp);      // dP = dO V^T
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const u32x4 draw = lds_read_b128(stat_addr + 256u + (uint32_t)(32 * qb + 8 * g) * 4u);
@@ -553,6 +594,25 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             }
             pp[2 * g] = N::pack2(v[0], v[1]);     // now dS, same operand order
             pp[2 * g + 1] = N::pack2(v[2], v[3]);
+        }
+        if (WRITE_DS) {
+            // Block (32-query block 2t + qb, this wave's 32-key block) of dS, 2 KiB, as the registers hold it: this
+            // lane's key against the queries 8g + 4*half + 0..3, g = 0..3.  Two store instructions of 1 KiB each,
+            // lane l writing bytes 16 l .. 16 l + 15 of its KiB: queries of g = 0, 1 in the first, g = 2, 3 in the second.
+            const long long block = (long long)bhk * fa_ds_blocks_per_head(S) + fa_ds_block_index(S, 2 * t + qb, kw >> 5);
+            // (Inline assembly: the block's address stays in two scalar registers and the lane's offset in one
+            // vector register that lives for these two instructions only -- as a 64-bit vector address it cost
+            // the registers that made the compiler spill inside the tile loop, and every reload from scratch
+            // memory there waits for all tile loads in flight.  Streaming stores: the blocks are read once, by
+            // another kernel, and should not displace the walked tiles from L2.  The wait states cover the rule
+            // that a store of more than 8 bytes must not be followed at once by a write of its data registers.)
+            const uint64_t dst = (uint64_t)(reinterpret_cast<char *>(a.ds_blocks) + block * kDsBlockBytes);
+            const uint64_t ub = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(dst >> 32)) << 32) |
+                                (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)dst);
+            const uint32_t voff = 16u * __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            const u32x4 w0 = {pp[0], pp[1], pp[2], pp[3]}, w1 = {pp[4], pp[5], pp[6], pp[7]};
+            asm volatile("global_store_dwordx4 %0, %1, %3 nt\n\tglobal_store_dwordx4 %0, %2, %3 offset:1024 nt\n\ts_nop 1"
+                         :: "v"(voff), "v"(w0), "v"(w1), "s"(ub) : "memory");
         }
 #pragma unroll
         for (int n = 0; n < 2 * DB; ++n) {                // dK^T += Q^T dS
@@ -580,26 +640,49 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
         wait_vm<0>();
 #pragma unroll
         for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
+        if (PARKED > 0) {           // from here on the last fragments live in LDS, and their registers are free
+            const uint32_t slot = park_lds + 32u * PARKED * (uint32_t)(wave * 64 + lane);
+#pragma unroll
+            for (int i = 0; i < PARKED; ++i) {
+                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + 32 * i) = kf[KS - PARKED + i];
+                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + 32 * i + 16) = vf[KS - PARKED + i];
+            }
+        }
         int stage = 0;
+        // WRITE_DS: the dS stores this wave made in the last two iterations, and the pairs still to come.  The next
+        // pair is then requested in front of an iteration's work instead of behind it.
+        int st1 = 0, st2 = 0, pairs_left = G * (t1 - t0 + 1);
+        constexpr bool TOP = WRITE_DS;
         for (int g = 0; g < G; ++g) {
             float slope_l2 = 0.0f;
             if (ALIBI) slope_l2 = a.alibi[hk * G + g] * kLog2e;
             for (int t = t1; t >= t0; --t) {
-                const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
+                const int next = stage == NSTG - 1 ? 0 : stage + 1, prev = stage == 0 ? NSTG - 1 : stage - 1;
                 const bool more = t - 1 >= t0 || g + 1 < G;
-                if (more) {                                     // this pair has landed, the next may still be in flight
+                --pairs_left;
+                if (WRITE_DS) {
+                    // This pair has landed when at most what was issued behind it is outstanding (memory operations
+                    // complete in the order they were issued): the loads of the pairs requested since, and the dS
+                    // stores made since.  Requests at the top of an iteration put a pair's loads in front of that
+                    // iteration's stores, so a store that takes long to be acknowledged holds up no load needed now.
+                    const int loads = wave < 2 ? 2 * IPW + 1 : 2 * IPW;     // waves 0 and 1 also fetch lse / delta
+                    wait_vm_upto((pairs_left > 0 ? loads : 0) + st1 + st2);
+                } else if (more) {                              // this pair has landed, the next may still be in flight
                     if (wave < 2) wait_vm<2 * IPW + 1>(); else wait_vm<2 * IPW>();     // waves 0 and 1 also fetch lse / delta
                 } else wait_vm<0>();
                 phase_barrier();
+                if (TOP && ig < G) issue_next(prev);
+                st2 = st1;
+                st1 = (WRITE_DS && my_lo <= t && t <= my_hi) ? 4 : 0;
                 if (my_lo <= t && t <= my_hi) {
                     const bool edge = MASKED && (fa_tile_class(64, Lq, Rq, kw, 32, t) == 1 || (GENERAL && (t + 1) * 64 > S));
                     const uint32_t bhq = (uint32_t)(b * a.H + hk * G + g);        // the head the forward keyed its dropout on
                     half_tile(edge, slope_l2, bhq, t, 0);
                     half_tile(edge, slope_l2, bhq, t, 1);
                 }
-                if (ig < G) issue_next(next == kBwdStages - 1 ? 0 : next + 1);
-                rd.advance(next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB);
-                stat_addr += next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB;
+                if (!TOP && ig < G) issue_next(prev);
+                rd.advance(next == 0 ? -(NSTG - 1) * STAGEB : STAGEB);
+                stat_addr += next == 0 ? -(NSTG - 1) * STAGEB : STAGEB;
                 stage = next;
             }
         }
@@ -636,6 +719,177 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     }   // next work item
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The five-product form (reference layout only).  fa_bwd_dq above and fa_bwd_dkdv each recompute S and dP: seven
+// products for five.  Here fa_bwd_dkdv, which has every dS block in registers as the operand of dK += dS^T Q,
+// also writes it out (WRITE_DS), and dQ = scale * dS K is one product over those blocks: every output element
+// still has exactly one writer and the same inputs give the same bits.  The price is S*S_kv storage-type elements
+// per head written once and read once, so this kernel is bound by HBM bandwidth, not by the matrix cores.
+//
+// fa_bwd_prepare: delta_i = sum_t dO_it O_it and the logsumexp in exp2 units, which fa_bwd_dkdv fetches per
+// query tile (fa_bwd_dq writes them in the seven-product form).
+// ---------------------------------------------------------------------------------------------------------
+template <bool BF16, int D>
+__global__ void __launch_bounds__(256) fa_bwd_prepare(const FaBwdArgs a)
+{
+    constexpr int TPR = D / 8;                    // threads per row, 16 bytes each
+    const long long row = (long long)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+    const long long n_rows = (long long)a.B * a.H * a.S;
+    const bool live = row < n_rows;
+    const long long r = live ? row : n_rows - 1;
+    const int c = (threadIdx.x % TPR) * 8;
+    const u32x4 o = *reinterpret_cast<const u32x4 *>(a.O + r * D + c);
+    const u32x4 g = *reinterpret_cast<const u32x4 *>(a.dO + r * D + c);
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t ow = o[w], gw = g[w];
+        sum += storage_to_f32<BF16>((uint16_t)(ow & 0xffffu)) * storage_to_f32<BF16>((uint16_t)(gw & 0xffffu));
+        sum += storage_to_f32<BF16>((uint16_t)(ow >> 16)) * storage_to_f32<BF16>((uint16_t)(gw >> 16));
+    }
+#pragma unroll
+    for (int m = 1; m < TPR; m <<= 1) sum += __shfl_xor(sum, m);
+    if (live && threadIdx.x % TPR == 0) {
+        a.delta[row] = sum;
+        const float l = a.lse[row];
+        a.lse2[row] = l == -INFINITY ? INFINITY : l * kLog2e;
+    }
+}
+
+// dQ^T += K^T dS^T over the dS blocks fa_bwd_dkdv<WRITE_DS> wrote.  A workgroup owns 256 queries (8 waves x one
+// 32-query block, lane = query) and walks the key tiles of its visible range.  LDS stage: the K tile (read
+// transposed, as in fa_bwd_dq) and, per wave, the two 2 KiB dS blocks of its query block against the tile's keys,
+// fetched by that wave alone.  A block comes in as it lies in memory except that the 64-byte groups of four keys
+// are XOR-permuted among the four 512-byte planes, so that the transposing read of a half-wave -- four keys, all
+// 32 queries, i.e. one group in each plane -- touches every LDS bank once.
+template <bool BF16, int D, bool MASKED>
+__global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaBwdArgs a)
+{
+    typedef Num<BF16> N;
+    typedef TileReader<D> Reader;
+    typedef TileLoader<D> Loader;
+    constexpr int DB = Reader::DB, TILEB = Loader::TILEB, IPW = Loader::IPW;
+    constexpr int WAVE_DS = 2 * kDsBlockBytes;                 // a wave's two blocks of a key tile
+    constexpr int STAGEB = TILEB + kBwdWaves * WAVE_DS;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int S = a.S;
+    const int n_qblocks = (S + 255) / 256;
+    const long long n_items = (long long)a.B * a.H * n_qblocks;
+    for (int pass = 0;; ++pass) {
+    const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
+    if (item >= n_items) break;
+    if (pass > 0) __syncthreads();          // (the LDS stages: other waves may still be reading the last tile)
+    int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(lane));
+    const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
+    int bh, qblock;
+    fa_item_decode(item, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
+    const uint16_t *Kh = a.K + (size_t)bh * S * D;
+    uint16_t *dQh = a.dQ + (size_t)bh * S * D;
+    const int q0 = qblock * 256, qw = q0 + wave * 32;
+    const bool active = qw < S;                    // the last block may own fewer than 256 rows
+    int t0, t1, my_lo = 1, my_hi = 0;
+    fa_tile_range(S, 64, a.L, a.R, q0, S - q0 < 256 ? S - q0 : 256, &t0, &t1);
+    if (active) fa_tile_range(S, 64, a.L, a.R, qw, 32, &my_lo, &my_hi);
+    // this head's dS blocks; this wave reads those of query block qw / 32
+    const char *ds_head = reinterpret_cast<const char *>(a.ds_blocks) + (long long)bh * fa_ds_blocks_per_head(S) * kDsBlockBytes;
+    const int my_qb = active ? qw >> 5 : 0;
+
+    Reader rd; rd.init(lane, lds0);
+    Loader ldk; ldk.init(wave, lane, D * 2);
+    // Source of the 16 bytes lane l brings in with instruction w (0, 1) of a block: LDS slot 64 w + l of the block
+    // = plane p = 2 w + l / 32, position l % 32; that position holds key ((l % 32 / 4) ^ p) * 4 + l % 4, which lies
+    // in memory at 1 KiB * w + 512 * (l / 32) + 16 * key.
+    uint32_t ds_src[2];
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+        const int p = 2 * w + half, key = ((((l32 >> 2) ^ p) & 7) << 2) | (l32 & 3);
+        ds_src[w] = (uint32_t)(1024 * w + 512 * half + 16 * key);
+    }
+    // Transposing read of a B operand (lane = query l32, keys 16 t2 + 4 half + {0..3} and + 8 of a block): the lane
+    // addresses the 8 bytes that hold queries 16 (l32 / 16) + 4 (l16 % 4) .. + 3 of key 16 t2 + 8 hi + 4 half + l16 / 4.
+    // Those four queries are quad 4 (l32 / 16) + l16 % 4 = 2 g + h of the block, written by fa_bwd_dkdv's lane
+    // (key, half h) as its g-th pair of words: plane p = 2 (g / 2) + h, 16-byte slot of the key, byte 8 (g % 2).
+    uint32_t ds_rd[2];
+    {
+        const int quad = 4 * (l32 >> 4) + (l16 & 3), g = quad >> 1, hq = quad & 1;
+        const int p = 2 * (g >> 1) + hq;
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+            ds_rd[hi] = lds0 + TILEB + wave * WAVE_DS +
+                        (uint32_t)(512 * p + ((((2 * hi + half) ^ p) & 3) << 6) + 16 * (l16 >> 2) + 8 * (g & 1));
+    }
+    auto issue = [&](int tile, int stage) __attribute__((always_inline)) {
+        const uint32_t base = lds0 + stage * STAGEB;
+        ldk.load(Kh + (size_t)tile * 64 * D, base);
+        if (my_lo <= tile && tile <= my_hi) {
+            const char *src = ds_head + fa_ds_block_index(S, my_qb, 2 * tile) * kDsBlockBytes;      // (and its neighbour 2 tile + 1)
+            const uint32_t dst = base + TILEB + wave * WAVE_DS;
+#pragma unroll
+            for (int n = 0; n < 4; ++n)         // block 2 tile (n = 0, 1), block 2 tile + 1 (n = 2, 3)
+                dma_16_stream(src, (uint32_t)((n >> 1) * kDsBlockBytes) + ds_src[n & 1], dst + n * 1024);
+        }
+    };
+    // the blocks fa_bwd_dkdv wrote: its wave with the 32 keys from `key0` on visits the query tiles of this range
+    auto block_written = [&](int key0) __attribute__((always_inline)) {
+        int lo, hi;
+        fa_tile_range(S, 64, a.R, a.L, key0, 32, &lo, &hi);
+        return lo <= (qw >> 6) && (qw >> 6) <= hi;
+    };
+
+    f32x16 dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) dq[db] = zero16();
+
+    if (t0 <= t1) {
+        issue(t0, 0);
+        if (t0 + 1 <= t1) issue(t0 + 1, 1);
+        wait_vm<0>();
+        int stage = 0;
+        for (int t = t0; t <= t1; ++t) {
+            const int next = stage == kBwdStages - 1 ? 0 : stage + 1;
+            if (t + 1 <= t1) {              // tile t has landed, tile t+1 may still be in flight
+                if (my_lo <= t + 1 && t + 1 <= my_hi) wait_vm<IPW + 4>(); else wait_vm<IPW>();
+            } else wait_vm<0>();
+            phase_barrier();
+            if (my_lo <= t && t <= my_hi) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    if (MASKED && !block_written(64 * t + 32 * kb)) continue;       // wave-uniform
+#pragma unroll
+                    for (int t2 = 0; t2 < 2; ++t2) {
+                        const u32x2 lo = lds_read_tr(ds_rd[0] + (uint32_t)(kb * kDsBlockBytes + 256 * t2));
+                        const u32x2 hi = lds_read_tr(ds_rd[1] + (uint32_t)(kb * kDsBlockBytes + 256 * t2));
+                        const u32x4 bfrag = {lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) dq[db] = N::mfma(rd.transposed(0, 2 * kb + t2, db), bfrag, dq[db]);
+                    }
+                }
+            }
+            if (t + 2 <= t1) issue(t + 2, next == kBwdStages - 1 ? 0 : next + 1);
+            const int delta = next == 0 ? -(kBwdStages - 1) * STAGEB : STAGEB;
+            rd.advance(delta);
+            ds_rd[0] += delta; ds_rd[1] += delta;
+            stage = next;
+        }
+    }
+    if (active) {
+        const int my_q = qw + l32;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                u32x2 w;
+                w[0] = N::pack2(dq[db][4 * g] * a.scale, dq[db][4 * g + 1] * a.scale);
+                w[1] = N::pack2(dq[db][4 * g + 2] * a.scale, dq[db][4 * g + 3] * a.scale);
+                *reinterpret_cast<u32x2 *>(dQh + (size_t)my_q * D + 32 * db + 8 * g + 4 * half) = w;
+            }
+    }
+    }   // next work item
+}
+
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
 hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream, bool configure_only = false)
 {
@@ -643,8 +897,12 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
     const unsigned grid_q = (unsigned)((long long)a.B * a.H * ((a.S + 255) / 256));
     const unsigned grid_k = (unsigned)((long long)a.B * a.Hk * ((a.Sk + 255) / 256));
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512) + (DROPOUT ? kBwdWaves * 128 : 0);
+    const int smem_dkdv_ds = kBwdStages * (2 * TILEB + 512) + (D == 128 ? 32 * kBwdWaves * 64 : 0);      // + the parked fragments
     auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
     auto kkv = fa_bwd_dkdv<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
+    // the five-product form: reference layout only
+    constexpr bool FIVE = LAYOUT == 0 && !ALIBI && !DROPOUT;
+    const int smem_dq_ds = kBwdStages * (TILEB + kBwdWaves * 2 * kDsBlockBytes);
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
     const unsigned long long dev_bit = 1ull << fa_launch_device();
@@ -653,6 +911,14 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
         if (e != hipSuccess) return e;
+        if constexpr (FIVE) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, 0, false, false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv_ds);
+            if (e != hipSuccess) return e;
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq_ds);
+            if (e != hipSuccess) return e;
+        }
         configured.fetch_or(dev_bit, std::memory_order_relaxed);
     }
     if (configure_only) return hipSuccess;     // (fa_init: the opt-in alone, so that no launch inside a stream capture makes it)
@@ -674,6 +940,17 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
     const bool uneven = LAYOUT == 0 && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
     const unsigned launch_q = (uneven && grid_q > resident && grid_q < 16u * resident) ? resident : grid_q;
     const unsigned launch_k = (uneven && grid_k > resident && grid_k < 16u * resident) ? resident : grid_k;
+    if constexpr (FIVE) {
+        if (a.ds_blocks != nullptr) {
+            // delta and the rescaled logsumexp; dK, dV and the dS blocks; dQ from the blocks
+            constexpr int rows_per_block = 256 / (D / 8);
+            const long long n_rows = (long long)a.B * a.H * a.S;
+            hipLaunchKernelGGL((fa_bwd_prepare<BF16, D>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, 0, false, false, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
+            hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL(kq, dim3(launch_q), dim3(kBwdWaves * 64), smem_dq, stream, a);
     hipLaunchKernelGGL(kkv, dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv, stream, a);
     return hipGetLastError();

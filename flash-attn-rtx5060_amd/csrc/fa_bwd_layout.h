@@ -48,4 +48,18 @@ FA_LAYOUT_HD int fa_bwd_tr_read(int D, int lane, int db, int hi)
     return row * D * 2 + ((c ^ fa_u_swz(cpr, row)) << 4) + ((c4 & 1) << 3);
 }
 
+// Where the 2 KiB dS block (32-query block qb, 32-key block kb) of a head lies in the five-product form's workspace,
+// in blocks from the head's start.  Blocks are grouped in squares of 8 x 8 (256 queries x 256 keys, 128 KiB): the
+// key-owning kernel (a workgroup = 8 key blocks, walking query tiles) and the query-owning kernel (a workgroup = 8
+// query blocks, walking key tiles) then each work through one contiguous 128 KiB square for four tiles in a row
+// (with whole block rows the query-owning kernel's eight waves read 512 KiB apart: 0.87 ms against 0.82 on B2 H32
+// S8192 D128); inside a square the key block runs fastest, so the two blocks a query-owning wave needs per key tile
+// are neighbours.
+FA_LAYOUT_HD long long fa_ds_squares_per_side(int S) { return (S / 32 + 7) / 8; }
+FA_LAYOUT_HD long long fa_ds_blocks_per_head(int S) { return fa_ds_squares_per_side(S) * fa_ds_squares_per_side(S) * 64; }
+FA_LAYOUT_HD long long fa_ds_block_index(int S, int qb, int kb)
+{
+    return (((long long)(qb >> 3) * fa_ds_squares_per_side(S) + (kb >> 3)) << 6) + ((qb & 7) << 3) + (kb & 7);
+}
+
 #endif

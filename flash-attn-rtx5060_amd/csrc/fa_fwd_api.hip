@@ -17,6 +17,7 @@
 #include "fa_fwd.h"
 #include "fa_bwd.h"
 #include "fa_bwd_args.h"
+#include "fa_bwd_layout.h"
 #include "fa_device_state.h"
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
@@ -604,6 +605,36 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
     return 2ull * (unsigned long long)p->B * p->N * p->S * 4ull;       // delta and the rescaled logsumexp
 }
 
+namespace {
+// the reference's layout and nothing else: contiguous [B,N,S,d], S a multiple of 128, as many keys and K/V heads,
+// no ALiBi, no dropout
+bool five_product_shape(const fa_bwd_params *p)
+{
+    if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S) || (p->n_kv_heads != 0 && p->n_kv_heads != p->N)) return false;
+    if (p->alibi_slopes_ptr != nullptr || p->dropout_prob > 0.0f) return false;
+    const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
+                                   p->dq_strides, p->dk_strides, p->dv_strides};
+    const long long dense[3] = {(long long)p->N * p->S * p->d, (long long)p->S * p->d, p->d};
+    for (int t = 0; t < 8; ++t) {
+        const long long *st = strides[t];
+        if (st[0] == 0 && st[1] == 0 && st[2] == 0) continue;
+        for (int k = 0; k < 3; ++k)
+            if (st[k] != dense[k]) return false;
+    }
+    return true;
+}
+unsigned long long ds_blocks_offset(const fa_bwd_params *p)
+{
+    return (fa_bwd_workspace_bytes(p) + 255ull) & ~255ull;
+}
+}  // namespace
+
+unsigned long long fa_bwd_fast_workspace_bytes(const fa_bwd_params *p)
+{
+    if (!p || p->B <= 0 || p->N <= 0 || p->S <= 0 || (p->d != 64 && p->d != 128) || !five_product_shape(p)) return 0;
+    return ds_blocks_offset(p) + (unsigned long long)p->B * p->N * (unsigned long long)fa_ds_blocks_per_head(p->S) * 2048ull;
+}
+
 int fa_bwd_validate(const fa_bwd_params *p)
 {
     if (!p || !p->Q || !p->K || !p->V || !p->O || !p->dO || !p->L || !p->dQ || !p->dK || !p->dV) return FA_ERR_NULL_POINTER;
@@ -656,6 +687,10 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.lse = p->L;
     a.delta = static_cast<float *>(p->workspace);
     a.lse2 = a.delta + (size_t)p->B * p->N * p->S;
+    // a workspace large enough for the dS blocks selects the five-product form
+    const unsigned long long fast_bytes = fa_bwd_fast_workspace_bytes(p);
+    a.ds_blocks = (fast_bytes != 0 && p->workspace_bytes >= fast_bytes)
+        ? reinterpret_cast<uint16_t *>(static_cast<char *>(p->workspace) + ds_blocks_offset(p)) : nullptr;
     a.dQ = static_cast<uint16_t *>(p->dQ);
     a.dK = static_cast<uint16_t *>(p->dK);
     a.dV = static_cast<uint16_t *>(p->dV);

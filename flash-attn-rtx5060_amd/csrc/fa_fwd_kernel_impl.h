@@ -48,6 +48,12 @@
 #include "fa_kernel_args.h"
 #include "fa_sched.h"
 
+// The row maximum of a tile's scores is taken next to this many of the iteration's first matrix instructions
+// (0: in front of them).
+#ifndef FA_ROW_MAX_SLOTS
+#define FA_ROW_MAX_SLOTS 4
+#endif
+
 namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -818,9 +824,17 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         if (DROPOUT) draw_dropout(tile);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
-        bool moved;
-        const float alpha = new_reference(row_max(), moved);
-        float nmc = -m_run * cs;
+        // The row maximum rides along with the first MAXG matrix instructions of PV(tile-1), which do not depend on
+        // it (a quarter of the 32 scores per lane each); the reference point moves behind the last of them, without
+        // a branch: a factor of exactly 1 where it stays.  The exponentials follow over the remaining instructions.
+        constexpr int MAXG = FA_ROW_MAX_SLOTS;
+        static_assert(MAXG == 0 || (16 % MAXG == 0 && MAXG < NPV), "row-maximum slots");
+        bool moved = false;
+        float alpha = 1.0f, nmc = 0.0f, mx = 0.0f;
+        if (MAXG == 0) {
+            alpha = new_reference(row_max(), moved);
+            nmc = -m_run * cs;
+        }
         uint32_t pn[16];                           // P(tile), becomes pk at the end
         f32x16 nx[2];                              // S^T(tile+1)
         __builtin_amdgcn_sched_barrier(0);
@@ -835,9 +849,32 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
                 const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 nx[n & 1] = N::mfma(fr[g], qf[n >> 1], n >= 2 ? nx[n & 1] : ALIBI ? alibi_start(n & 1, tile + 1) : zero);
             }
-            // softmax work riding along: the 16 element pairs of this tile spread over the NF matrix instructions
+            if (g < MAXG) {
+                constexpr int PER = MAXG > 0 ? 16 / MAXG : 16;
+                if (g == 0) mx = max_plain(sx[0][0], sx[1][0]);
+                asm volatile("" : "+v"(mx));
+#pragma unroll
+                for (int r = g * PER + (g == 0 ? 1 : 0); r < (g + 1) * PER; ++r) mx = fmaxf(fmaxf(mx, sx[0][r]), sx[1][r]);
+                if (g == MAXG - 1) {
+                    mx = max_of_halves(mx);
+                    const bool grow = mx > m_run + thresh;      // (from kNoReference every finite maximum grows)
+                    moved = __builtin_amdgcn_ballot_w64(grow) != 0;
+                    const float m_new = grow ? mx : m_run;
+                    alpha = __builtin_amdgcn_exp2f((m_run - m_new) * cs);
+                    l_a *= alpha;
+                    l_b *= alpha;
+                    m_run = m_new;
+                    nmc = -m_new * cs;
+                    asm volatile("" : "+v"(nmc), "+v"(l_a), "+v"(l_b));
+                } else {
+                    asm volatile("" : "+v"(mx));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
+            }
+            // softmax work riding along: the 16 element pairs of this tile spread over the matrix instructions
             constexpr int PAIRS = 16;
-            const int p_begin = (g * PAIRS) / NF, p_end = ((g + 1) * PAIRS) / NF;
+            const int p_begin = ((g - MAXG) * PAIRS) / (NF - MAXG), p_end = ((g - MAXG + 1) * PAIRS) / (NF - MAXG);
 #pragma unroll
             for (int e = p_begin; e < p_end; ++e) {
                 // pair e: elements (2e, 2e+1) of key block 0 for e < 8, of key block 1 for e >= 8.  The two empty

@@ -37,7 +37,8 @@ typedef struct fa_bwd_params {
     int window_size_right;
     int dtype;                /* FA_DTYPE_F16 / FA_DTYPE_BF16                                                  */
     int is_causal;
-    void *workspace;          /* device scratch, at least fa_bwd_workspace_bytes(): 2*B*N*S floats               */
+    void *workspace;          /* device scratch, at least fa_bwd_workspace_bytes(): 2*B*N*S floats; with at least
+                                 fa_bwd_fast_workspace_bytes() (when that is not 0) the five-product form runs   */
     unsigned long long workspace_bytes;
     /* ---- general layouts; all zero = the reference's contiguous [B,N,S,d] with S_kv = S ---- */
     int n_kv_heads;           /* 0 = N; otherwise divides N                                                    */
@@ -57,8 +58,15 @@ typedef struct fa_bwd_params {
 
 int fa_bwd_validate(const fa_bwd_params *p);
 unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p);
-/* Enqueues two kernels on `stream` (dQ and the row sums of dO*O, then dK and dV) and returns without
- * synchronising.  No atomics: the same inputs give the same bits on every run. */
+/* The workspace size that selects the five-product form, or 0 when the problem is not the reference's layout
+ * (contiguous [B,N,S,d], S a multiple of 128, as many keys and K/V heads, no ALiBi, no dropout): the small
+ * workspace plus B*N*S*S storage-type elements (c3's shape: 8.6 GB).  With it, the key-owning kernel writes every
+ * dS block it forms and dQ is one product over those blocks, instead of a second recomputation of S and dP. */
+unsigned long long fa_bwd_fast_workspace_bytes(const fa_bwd_params *p);
+/* Enqueues the backward pass on `stream` and returns without synchronising: two kernels (dQ and the row sums of
+ * dO*O, then dK and dV: seven matrix products), or, with the large workspace, three (the row sums; dK, dV and the
+ * dS blocks; dQ from the blocks: five products).  No atomics either way: every output element has one writer and
+ * the same inputs give the same bits on every run. */
 int fa_bwd(const fa_bwd_params *p, void *stream);
 /* Host mirror of the arithmetic with which the key-owning kernel finds its work (csrc/fa_sched.h with the two
  * sides of the mask exchanged and shifted by S_kv - S): the inclusive range of 64-query tiles that contain a

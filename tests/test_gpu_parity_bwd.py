@@ -51,12 +51,77 @@ def test_gradients_against_the_fp64_oracle(fa, oracle, shape, dtype, causal, wl,
     dq_ref, dk_ref, dv_ref = oracle.bwd_f64(q, k, v, do, dtype, None, causal, wl, wr)
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
     o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, exact_first_rows=True)
-    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr)
+    # (the seven-product form: fa_bwd_dq and fa_bwd_dkdv; the five-product form has its own test below)
+    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=False)
     torch.cuda.synchronize()
     for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
         err = grad_errors(oracle.to_f32(from_torch(got), dtype), want)
         print(shape, dtype, causal, wl, wr, name, err, flush=True)
         check(err, dtype, name)
+
+
+FIVE_CASES = [
+    # shape, dtype, causal, wl, wr: the reference's layout (S a multiple of 128), every kind of band
+    ((1, 2, 128, 64), 0, False, -1, -1),
+    ((2, 2, 256, 128), 0, True, -1, -1),
+    ((1, 2, 384, 64), 1, True, -1, -1),
+    ((1, 2, 640, 128), 0, True, 100, -1),
+    ((1, 2, 512, 64), 0, False, 70, 50),
+    ((1, 2, 512, 128), 0, False, -1, 32),      # a right window that ends on a 32-key block edge
+    ((1, 2, 512, 128), 1, False, -1, 33),
+    ((1, 1, 384, 64), 0, False, 31, 0),
+    ((1, 1, 384, 128), 0, False, 0, 0),        # the diagonal alone
+    ((1, 2, 768, 128), 1, False, 128, 0),
+    ((1, 2, 1024, 128), 0, False, 5, 200),
+]
+
+
+@pytest.mark.parametrize("shape,dtype,causal,wl,wr", FIVE_CASES)
+def test_five_product_form_against_the_fp64_oracle(fa, oracle, shape, dtype, causal, wl, wr):
+    """fa_bwd with the large workspace (fa_bwd_fast_workspace_bytes): the key-owning kernel writes its dS blocks and
+    dQ is one product over them.  Through the C ABI, with the workspace filled with NaN beforehand: a block read
+    without having been written (the two kernels must agree on which blocks exist under every mask) poisons dQ."""
+    import ctypes
+    import torch
+    B, H, S, D = shape
+    q, k, v = make_inputs(fa, shape, dtype, seed=700 + S)
+    do, _, _ = make_inputs(fa, shape, dtype, seed=701 + S)
+    dq_ref, dk_ref, dv_ref = oracle.bwd_f64(q, k, v, do, dtype, None, causal, wl, wr)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, exact_first_rows=True)
+    dq, dk, dv = (torch.full_like(tq, float("nan")) for _ in range(3))
+    p = fa.make_bwd_params(B, H, S, D, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(), tdo.data_ptr(), lse.data_ptr(),
+                           dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), causal=causal, window_left=wl, window_right=wr, dtype=dtype)
+    L = fa.lib()
+    small, need = L.fa_bwd_workspace_bytes(ctypes.byref(p)), L.fa_bwd_fast_workspace_bytes(ctypes.byref(p))
+    assert need >= small + B * H * S * S * 2
+    ws = torch.full((need // 4 + 1,), float("nan"), dtype=torch.float32, device="cuda")
+    p.workspace, p.workspace_bytes = ws.data_ptr(), need
+    assert L.fa_bwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == fa.FA_OK
+    torch.cuda.synchronize()
+    for name, got, want in (("dQ", dq, dq_ref), ("dK", dk, dk_ref), ("dV", dv, dv_ref)):
+        err = grad_errors(oracle.to_f32(from_torch(got), dtype), want)
+        print("five products", shape, dtype, causal, wl, wr, name, err, flush=True)
+        check(err, dtype, name)
+    # the same bits on a second run
+    dq2, dk2, dv2 = (torch.full_like(tq, float("nan")) for _ in range(3))
+    p.dQ, p.dK, p.dV = dq2.data_ptr(), dk2.data_ptr(), dv2.data_ptr()
+    ws.fill_(float("nan"))
+    assert L.fa_bwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == fa.FA_OK
+    torch.cuda.synchronize()
+    for a_, b_ in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.equal(a_.view(torch.int16), b_.view(torch.int16))
+
+
+def test_five_product_workspace_is_offered_for_the_reference_layout_only(fa):
+    import ctypes
+    L = fa.lib()
+    ok = dict(B=2, N=4, S=1024, d=128)
+    small = L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok)))
+    assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == ((small + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
+    for other in (dict(S=1000), dict(S_kv=2048), dict(n_kv_heads=2), dict(dropout_prob=0.1), dict(alibi_ptr=256),
+                  dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)})):
+        assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
@@ -188,7 +253,8 @@ def test_general_layouts_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D
 @pytest.mark.parametrize("D,dtype,causal,wl", [(128, 0, True, -1), (64, 1, False, -1), (128, 1, True, 200), (64, 0, True, -1)])
 def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl):
     """[B,S,H,D] storage goes through the strided kernels, [B,H,S,D] through the plain ones: same values, same
-    arithmetic in the same order, so dQ, dK and dV have to agree bit for bit."""
+    arithmetic in the same order, so dQ, dK and dV have to agree bit for bit.  (The seven-product form, which is the
+    only one the strided layout has; the five-product form of the reference's layout sums in another order.)"""
     import torch
     B, H, S = 2, 3, 768
     q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed=910 + D)
@@ -198,7 +264,7 @@ def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl)
     got = []
     for tq, tk, tv, tdo in (dense, bshd):
         o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl)
-        got.append(fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl))
+        got.append(fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, five_products=False))
     torch.cuda.synchronize()
     assert got[1][0].stride() == bshd[0].stride()
     for name, a, b in zip(("dQ", "dK", "dV"), got[0], got[1]):
