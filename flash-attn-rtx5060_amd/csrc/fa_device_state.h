@@ -14,6 +14,9 @@ struct FaDeviceState {
     unsigned *queues;          // kFaQueueSlots sets of 16 words (nine used)
     unsigned char *scratch;    // kFaStaticScratchBytes bytes, 256-byte aligned
     int compute_units;
+#ifdef FA_CHECK_RING
+    unsigned long long *ring_check;     // checking build: comparisons made, mismatches found
+#endif
 };
 
 // State of the current device (set up on first use).  Also records the device index for fa_launch_device().

@@ -435,6 +435,9 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
     a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
     a.seed_hi = (unsigned)(p->seed >> 32);
     a.exact_first_rows = p->exact_first_rows != 0;
+#ifdef FA_CHECK_RING
+    a.ring_check = ds->ring_check;
+#endif
     hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general
                     : strided ? fa_launch_forward_strided : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
@@ -487,6 +490,26 @@ int fa_fwd_split_static(const fa_fwd_params *p, void *stream)
     // the kernels get the array's device address, exactly as they get a caller's workspace in fa_fwd
     return forward(p, ds->scratch, ds, stream);
 }
+
+#ifdef FA_CHECK_RING
+// Checking build only (libfa_fwd_gfx950_check.so): waits for the device, returns how many 16-byte comparisons the
+// forward kernels' ring checks have made and how many of them found other bytes in LDS than the tile the
+// iteration expected, and sets both counters back to zero.
+int fa_debug_ring_counts(unsigned long long *checks, unsigned long long *violations)
+{
+    const FaDeviceState *ds = nullptr;
+    hipError_t e = fa_device_state(&ds);
+    if (e != hipSuccess) return device_fail(e, "device set-up");
+    unsigned long long host[2] = {0, 0};
+    e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemcpy(host, ds->ring_check, sizeof(host), hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemset(ds->ring_check, 0, sizeof(host));
+    if (e != hipSuccess) return device_fail(e, "ring check counters");
+    if (checks) *checks = host[0];
+    if (violations) *violations = host[1];
+    return FA_OK;
+}
+#endif
 
 int fa_reset_work_queues(void)
 {

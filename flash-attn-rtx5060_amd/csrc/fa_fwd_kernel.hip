@@ -16,6 +16,10 @@ static __device__ __align__(256) unsigned g_work_queues[kFaQueueSlots][16];
 // In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
 static __device__ __align__(256) unsigned char g_split_scratch[kFaStaticScratchBytes];
 
+#ifdef FA_CHECK_RING
+static __device__ __align__(16) unsigned long long g_ring_check[2];
+#endif
+
 namespace {
 std::mutex g_state_mutex;
 FaDeviceState g_state[kFaMaxDevices] = {};
@@ -39,6 +43,10 @@ hipError_t fa_device_state(const FaDeviceState **state)
             e = hipGetSymbolAddress(reinterpret_cast<void **>(&st.scratch), HIP_SYMBOL(g_split_scratch));
             if (e != hipSuccess) return e;
             if (st.queues == nullptr || st.scratch == nullptr) return hipErrorInvalidSymbol;
+#ifdef FA_CHECK_RING
+            e = hipGetSymbolAddress(reinterpret_cast<void **>(&st.ring_check), HIP_SYMBOL(g_ring_check));
+            if (e != hipSuccess) return e;
+#endif
             int n = 0;
             e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
             if (e != hipSuccess) return e;

@@ -925,29 +925,62 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     // Every wave executes every iteration (one barrier each); a wave whose own tile range does not cover all
     // three pieces runs the plain pieces it has, the others run the interleaved body.  The two kinds live in
     // separate loops: merging them under one branch makes the register allocator spill.
-    bool prev_full = false;     // the previous iteration requested both of its tiles
     auto finish_iteration = [&](bool full_issue, bool past_last_request) __attribute__((always_inline)) {
         // What the next iteration reads must have landed: that was requested LA - 1 iterations ago, so the
         // requests of the LA - 1 most recent iterations may stay in flight (vmcnt counts requests, so this only
         // holds while every one of those iterations made all of its 2 * IPW requests)
-        if (NST == 4 && full_issue && prev_full) wait_vm<4 * IPW>();
-        else if (NST >= 3 && full_issue) wait_vm<2 * IPW>();
+        if (NST >= 3 && full_issue) wait_vm<2 * IPW>();
         // (the last iterations of an item, those past the request for V(t1), request nothing, and the one before
         // them has waited for everything: they do not wait, so that the counter fetched there for the next
         // item stays in flight)
         else if (!past_last_request) wait_vm<0>();
-        prev_full = full_issue;
         phase_barrier();
     };
+#ifdef FA_CHECK_RING
+    // Checking build: the invariants of the LDS ring, asserted by every wave in every iteration.  In front of the
+    // iteration's work and again behind it (in front of the barrier that releases the stages), K stage `kstage` must
+    // hold key tile i + 1 and V stage `vstage` key tile i - 1: each lane compares sixteen bytes of both stages with
+    // the same bytes read from global memory.  A tile that has not landed when it is read (a wait that counts too
+    // few requests, a missing barrier) or that is overwritten while others still read it (a request issued a stage
+    // too early) shows up as a mismatch; nothing traps, the counters are read by the host afterwards.
+    auto ring_check = [&](int i, int kstage, int vstage, int salt) __attribute__((always_inline)) {
+        const int row = lane, chunk = (wave + salt) % CPR;          // one 16-byte chunk per lane
+        unsigned long long checked = 0, bad = 0;
+        for (int which = 0; which < 2; ++which) {
+            const int tile = which == 0 ? i + 1 : i - 1;
+            if (tile < t0 || tile > t1) continue;
+            const int key = tile * kBlockKeys + row;
+            if (key >= Sk) continue;                                 // (GENERAL: rows past the end hold copies of the last row)
+            const int swz = which == 0 ? k_swz<CPR>(row) : v_swz<CPR>(row);
+            const uint32_t addr = lds0 + (which == 0 ? 0u : LDS_V) + (uint32_t)((which == 0 ? kstage : vstage) * TILEB + row * ROWB + ((chunk ^ swz) << 4));
+            const u32x4 in_lds = lds_read_b128(addr);
+            const uint16_t *src = (which == 0 ? Kh + (size_t)key * k_rs : Vh + (size_t)key * v_rs) + 8 * chunk;
+            const u32x4 in_mem = *reinterpret_cast<const u32x4 *>(src);
+            ++checked;
+            if (in_lds[0] != in_mem[0] || in_lds[1] != in_mem[1] || in_lds[2] != in_mem[2] || in_lds[3] != in_mem[3]) ++bad;
+        }
+        // (the compiler's wait for the global loads above is a wait for every request in flight: it can only hide a
+        // violation that would have happened after this point, never produce one)
+        if (a.ring_check != nullptr) {
+            if (checked) atomicAdd(&a.ring_check[0], checked);
+            if (bad) atomicAdd(&a.ring_check[1], bad);
+        }
+    };
+#define FA_RING_CHECK(i, ks, vs, salt) ring_check(i, ks, vs, salt)
+#else
+#define FA_RING_CHECK(i, ks, vs, salt) do { } while (0)
+#endif
     auto generic_iteration = [&](int i, int j3) __attribute__((always_inline)) {
         const int tk = i + 1 + LA, tv = i - 1 + LA;
         const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
         const int jm1 = j3 == 0 ? NST - 1 : j3 - 1, jm2 = jm1 == 0 ? NST - 1 : jm1 - 1, jm3 = jm2 == 0 ? NST - 1 : jm2 - 1;
         if (more_k) issue_k(tk, jm1);              // (j + LA) % NST == (j - 1) % NST
         if (more_v) issue_v(tv, jm3);              // (j - 2 + LA) % NST == (j - 3) % NST
+        FA_RING_CHECK(i, j3, jm2, 0);
         if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(jm2);
         if (my_lo <= i && i <= my_hi) softmax_plain(i);
         if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3, i + 1);
+        FA_RING_CHECK(i, j3, jm2, 3);
         finish_iteration(more_k && more_v, tv > t1);
     };
     auto steady_iteration = [&](auto J3, int i) __attribute__((always_inline)) {
@@ -955,9 +988,16 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         constexpr int jm1 = (j3 + NST - 1) % NST, jm2 = (j3 + 2 * NST - 2) % NST, jm3 = (j3 + 3 * NST - 3) % NST;
         const int tk = i + 1 + LA, tv = i - 1 + LA;
         const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
+#ifdef FA_CHECK_RING_BREAK
+        // the checker's negative control: the K tile goes into the stage that is being read in this iteration
+        if (more_k) issue_k(tk, j3);
+#else
         if (more_k) issue_k(tk, jm1);
+#endif
         if (more_v) issue_v(tv, jm3);
+        FA_RING_CHECK(i, j3, jm2, 1);
         steady(IntC<j3>{}, IntC<jm2>{}, i);
+        FA_RING_CHECK(i, j3, jm2, 5);
         finish_iteration(more_k && more_v, false);
     };
     int i = t0 - 1, j3 = 0;

@@ -42,6 +42,10 @@ struct FaKernelArgs {
     unsigned seed_lo, seed_hi;
     // --- masked instantiations
     int exact_first_rows;      // 1: no row is recomputed in the reference verifier's rounded-product arithmetic
+#ifdef FA_CHECK_RING
+    // checking build only: [0] comparisons made, [1] LDS bytes that were not the tile the iteration expected
+    unsigned long long *ring_check;
+#endif
 };
 
 #endif
