@@ -30,6 +30,8 @@ hipError_t fa_launch_forward_general(const FaKernelArgs &a, int bf16, int D, int
                                      hipStream_t stream);
 hipError_t fa_launch_forward_dropout(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
                                      hipStream_t stream);
+hipError_t fa_launch_forward_dropout_regular(const FaKernelArgs &a, int bf16, int D, int masked, int shape, unsigned grid,
+                                             hipStream_t stream);
 hipError_t fa_launch_combine_splits(const FaKernelArgs &a, int bf16, int D, hipStream_t stream);
 hipError_t fa_launch_backward(const FaBwdArgs &a, int bf16, int D, int masked, int general, int alibi, int compute_units,
                               hipStream_t stream, bool configure_only = false);
@@ -42,6 +44,7 @@ hipError_t fa_configure_forward_contiguous();
 hipError_t fa_configure_forward_strided();
 hipError_t fa_configure_forward_general();
 hipError_t fa_configure_forward_dropout();
+hipError_t fa_configure_forward_dropout_regular();
 hipError_t fa_configure_backward();
 hipError_t fa_configure_backward_dropout();
 hipError_t fa_configure_backward_strided();
@@ -438,7 +441,8 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
 #ifdef FA_CHECK_RING
     a.ring_check = ds->ring_check;
 #endif
-    hipError_t e = (a.drop_threshold != 0 ? fa_launch_forward_dropout : general ? fa_launch_forward_general
+    hipError_t e = (a.drop_threshold != 0 ? (general ? fa_launch_forward_dropout : fa_launch_forward_dropout_regular)
+                    : general ? fa_launch_forward_general
                     : strided ? fa_launch_forward_strided : fa_launch_forward_contiguous)(
         a, p->dtype == FA_DTYPE_BF16, p->d, masked, shape, (unsigned)grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return device_fail(e, "forward launch");
@@ -458,7 +462,7 @@ int fa_init(void)
     // everything a first launch would otherwise do besides the launch itself: after this call no entry point makes
     // a HIP call on this device that is not a stream operation (which is what a stream capture needs)
     hipError_t (*const configure[])() = {fa_configure_forward_contiguous, fa_configure_forward_strided, fa_configure_forward_general,
-                                         fa_configure_forward_dropout, fa_configure_backward, fa_configure_backward_dropout,
+                                         fa_configure_forward_dropout, fa_configure_forward_dropout_regular, fa_configure_backward, fa_configure_backward_dropout,
                                          fa_configure_backward_strided};
     for (auto fn : configure) {
         e = fn();

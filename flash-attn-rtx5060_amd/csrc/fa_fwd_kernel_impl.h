@@ -189,8 +189,10 @@ __device__ __forceinline__ DropWords dropout_words(uint32_t seed_lo, uint32_t se
     uint32_t c0 = group, c1 = i, c2 = bh, c3 = 0x44524F50u, k0 = seed_lo, k1 = seed_hi;
 #pragma unroll
     for (int round = 0; round < 10; ++round) {
-        const uint32_t h0 = __umulhi(0xD2511F53u, c0), l0 = 0xD2511F53u * c0;
-        const uint32_t h1 = __umulhi(0xCD9E8D57u, c2), l1 = 0xCD9E8D57u * c2;
+        // (one 32 x 32 -> 64-bit multiply-add instruction per product instead of a high and a low multiply, each
+        // of which runs at a quarter of the vector ALU's rate)
+        const uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c0, p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
+        const uint32_t h0 = (uint32_t)(p0 >> 32), l0 = (uint32_t)p0, h1 = (uint32_t)(p1 >> 32), l1 = (uint32_t)p1;
         c0 = h1 ^ c1 ^ k0; c1 = l1; c2 = h0 ^ c3 ^ k1; c3 = l0;
         k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
     }
@@ -349,7 +351,10 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
             pj = ex[e] / rsum[i];
             if (drop_threshold != 0u) {        // keys 0..31: one 32-key block, two Philox blocks per query
                 const DropWords d = dropout_words(seed_lo, seed_hi, bh, (uint32_t)(i + pos_off), (uint32_t)((j >> 2) & 1));
-                pj = dropout_keep_byte(d, 4 * (j >> 3) + (j & 3), drop_threshold) ? __fmul_rn(pj, drop_scale) : 0.0f;
+                // (the word is picked with selects: indexed with a run-time value the four words would live in scratch memory)
+                const int wi = j >> 3;
+                const uint32_t word = wi == 0 ? d.w[0] : wi == 1 ? d.w[1] : wi == 2 ? d.w[2] : d.w[3];
+                pj = ((word >> (8 * (j & 3))) & 255u) >= drop_threshold ? __fmul_rn(pj, drop_scale) : 0.0f;
             }
         }
         const uint32_t bits = f32_to_storage<BF16>(pj);
@@ -821,6 +826,9 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         };
 #pragma unroll
         for (int n = 0; n < PD; ++n) fetch(n);
+        // (Dropout: the tile's two Philox blocks are drawn here, in one piece.  Spread over the first ten matrix
+        // instructions, two rounds each, they measured 1-5 % slower: with dropout the iteration is bound by the
+        // vector ALU, not by the matrix pipe it would be hiding behind.)
         if (DROPOUT) draw_dropout(tile);
         // the fragments are in flight; the row maxima need no matrix instruction and cover their latency
         if (MASKED && tile_class(tile) == 1) apply_mask(tile);
