@@ -25,8 +25,10 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 MEASURED_HBM_BYTES = {"c3": 573.9e6, "c2": 68.2e6, "c4": 780.4e6}
 TRAFFIC_SOURCE = {"c3": "profiles/fa_fwd_pipelined_c3_pmc.md", "c2": "profiles/fa_fwd_pipelined_c2_pmc.md",
                   "c4": "profiles/fa_fwd_pipelined_c4_pmc.md"}
-# the same for the two backward kernels together on c3's shape: 1756.4 MB read + 414.9 MB written
-MEASURED_BWD_HBM_BYTES = {"c3": 2171.3e6}
+# the same for the backward kernels together on c3's shape (profiles/fa_bwd_c3_backward.md): the five-product form
+# 5692.6 MB read + 4762.8 MB written (8.6 GB of it the dS blocks, written once and read once), the seven-product
+# form 1756.4 MB read + 414.9 MB written
+MEASURED_BWD_HBM_BYTES = {"c3": {"five": 10455.4e6, "seven": 2171.3e6}}
 
 WORKLOADS = {
     # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
@@ -105,7 +107,7 @@ def decode_bench(args):
 
 
 def backward_bench(args):
-    """One JSON line for the backward pass (fa_bwd: dQ with the row sums of dO*O, then dK and dV) on a forward workload's shape:
+    """One JSON line for the backward pass (fa_bwd; --bwd-form picks the five- or the seven-product form) on a forward workload's shape:
     a step is one backward pass over the whole batch; FLOPs are 2.5 x the forward's (five products over the
     unmasked pairs instead of two).  Parity: one head against torch's fp32 attention and autograd on the GPU
     (the fp64 gradient oracle checks small shapes in tests/)."""
@@ -169,6 +171,8 @@ def backward_bench(args):
         d = got[-1, -1].float() - want
         err[name] = {"rel_l2": float(d.norm() / want.norm()), "max_abs": float(d.abs().max()), "max_ref": float(want.abs().max())}
     tf = flops / (wall_ms * 1e-3) / 1e12
+    plain = args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads and not args.alibi      # the reference's layout
+    form = "five" if (args.bwd_form == "five" and plain) else "seven"
     print(json.dumps({
         "metric": "attn backward TFLOPS (dQ, dK, dV), 1 GPU", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
@@ -181,8 +185,9 @@ def backward_bench(args):
                    "seed": seed, "algorithmic_flops": flops},
         "roofline": {"bound": "mfma", "achieved": round(flops / (gpu_ms * 1e-3) / 1e12, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (gpu_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload) if args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads and not args.alibi else None,
-                     "kernel_ms_avg": round(gpu_ms, 5), "kernels": "fa_bwd_dq + fa_bwd_dkdv"},
+                     "traffic": MEASURED_BWD_HBM_BYTES.get(args.workload, {}).get(form) if plain else None,
+                     "kernel_ms_avg": round(gpu_ms, 5),
+                     "kernels": "fa_bwd_prepare + fa_bwd_dkdv (writes dS) + fa_bwd_dq_from_ds" if form == "five" else "fa_bwd_dq + fa_bwd_dkdv"},
         "parity_vs_torch_fp32_one_head": err}))
 
 
@@ -357,21 +362,26 @@ def main():
         rng = np.random.default_rng(seed)
         # size the sample from a probe large enough that the per-head set-up (K and V widened once per head
         # touched) no longer dominates its time
-        probe = np.sort(rng.choice(B * H * S, size=min(B * H * S, 4096), replace=False))
-        t = time.perf_counter()
-        ob.rows(q, kf, vf, probe, dtype, None, causal, wl, -1, slopes, threads=cores, dropout=drop)
-        per_row = max((time.perf_counter() - t) / len(probe), 1e-7)
-        n = int(min(B * H * S, max(len(probe), 0.5 * args.cpu_seconds / per_row)))
-        spent = 0.0
-        for attempt in range(2):    # (one resize if the first sample came out short; both together stay near the target)
-            sample = np.sort(rng.choice(B * H * S, size=n, replace=False))
-            t = time.perf_counter()
-            ob.rows(q, kf, vf, sample, dtype, None, causal, wl, -1, slopes, threads=cores, dropout=drop)
-            dt = time.perf_counter() - t
-            spent += dt
-            if dt >= 0.4 * args.cpu_seconds or n >= B * H * S:
-                break
-            n = int(min(B * H * S, n * max(args.cpu_seconds - spent, 0.0) / max(dt, 1e-3)))
+        total = B * H * S
+
+        def timed_rows(n_rows):
+            rows_ = np.sort(rng.choice(total, size=n_rows, replace=False))
+            t_ = time.perf_counter()
+            ob.rows(q, kf, vf, rows_, dtype, None, causal, wl, -1, slopes, threads=cores, dropout=drop)
+            return rows_, time.perf_counter() - t_
+        # The cost of a sample is a fixed part (K and V widened once per head touched) plus a part per row: two small
+        # samples give both, and the third is sized so that all three together stay near the target.
+        n1, n2 = min(total, 4096), min(total, 32768)
+        _, t1 = timed_rows(n1)
+        sample, dt = timed_rows(n2)
+        n = n2
+        if n2 > n1:
+            per_row = max((dt - t1) / (n2 - n1), 1e-8)
+            fixed = max(dt - per_row * n2, 0.0)
+            want = int((args.cpu_seconds - t1 - dt - fixed) / per_row)
+            if want > 2 * n2:
+                n = min(total, want)
+                sample, dt = timed_rows(n)
         pairs = 0
         for r in sample.tolist():
             i = r % S

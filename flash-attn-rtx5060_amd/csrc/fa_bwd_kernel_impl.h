@@ -509,11 +509,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // stores in flight.  The last PARKED of the K^T and V^T fragments, which every half tile uses once, are kept in
     // LDS instead (32 bytes per lane and fragment pair, written once per work item) and read like any A operand.
     constexpr int PARKED = WRITE_DS && D == 128 ? 1 : 0;
+    constexpr uint32_t kParkPlane = 16u * kBwdWaves * 64u;
     const uint32_t park_lds = lds0 + NSTG * STAGEB;
     auto parked = [&](int which, int s) __attribute__((always_inline)) {
         uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
         asm volatile("" : "+v"(ln));
-        const uint32_t addr = park_lds + 32u * PARKED * ((uint32_t)wave * 64u + ln) + 32u * (uint32_t)(s - (KS - PARKED)) + 16u * which;
+        const uint32_t addr = park_lds + 16u * ((uint32_t)wave * 64u + ln) + kParkPlane * (uint32_t)(2 * (s - (KS - PARKED)) + which);
         return *(volatile __attribute__((address_space(3))) u32x4 *)(uintptr_t)addr;
     };
 
@@ -641,11 +642,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
 #pragma unroll
         for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
         if (PARKED > 0) {           // from here on the last fragments live in LDS, and their registers are free
-            const uint32_t slot = park_lds + 32u * PARKED * (uint32_t)(wave * 64 + lane);
+            // (one plane of 16 bytes per thread for every parked fragment: consecutive lanes, consecutive 16 bytes)
+            const uint32_t slot = park_lds + 16u * (uint32_t)(wave * 64 + lane);
 #pragma unroll
             for (int i = 0; i < PARKED; ++i) {
-                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + 32 * i) = kf[KS - PARKED + i];
-                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + 32 * i + 16) = vf[KS - PARKED + i];
+                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + kParkPlane * (2 * i)) = kf[KS - PARKED + i];
+                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)(slot + kParkPlane * (2 * i + 1)) = vf[KS - PARKED + i];
             }
         }
         int stage = 0;
