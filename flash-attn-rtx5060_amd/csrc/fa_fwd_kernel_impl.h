@@ -50,6 +50,10 @@
 
 // The row maximum of a tile's scores is taken next to this many of the iteration's first matrix instructions
 // (0: in front of them).
+#ifndef FA_S1K
+#define FA_S1K 3
+#define FA_S1V 2
+#endif
 #ifndef FA_ROW_MAX_SLOTS
 #define FA_ROW_MAX_SLOTS 4
 #endif
@@ -401,7 +405,7 @@ __device__ __forceinline__ void faithful_first_rows(const uint16_t *Qh, const ui
 // ---------------------------------------------------------------------------
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false, int NSTV = NST>
 __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArgs a)
 {
     constexpr int WR = 32;                        // query rows per wave
@@ -417,13 +421,16 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     constexpr int NQK = 2 * KS;                   // K fragments per tile: (head-dim slice, 32-key block)
     constexpr int NF = NPV + NQK;                 // every fragment feeds one matrix instruction
     constexpr int PD = 6;                         // LDS reads run this many fragments ahead
-    constexpr int LA = NST - 1;                   // tiles are loaded LA iterations before their first use
+    constexpr int LA = NST - 1;                   // K tiles are requested LA iterations before their first use
+    constexpr int LAV = NSTV - 1;                 // V tiles likewise (NSTV V stages: as many as K stages, or one fewer)
+    constexpr int STAGES = NST + NSTV;
     // (the first-rows path works in LDS behind the K stages that the requests for the next item fill)
-    static_assert(GENERAL || LA * TILEB + NW * 32 * ROWB <= 2 * NST * TILEB, "the epilogue's row blocks do not fit behind the requested stages");
-    static_assert(NST <= 3 && LA * TILEB + 3 * kFaithfulRows * D * 2 + 2 * 4096 + 128 <= 2 * NST * TILEB, "first-rows path does not fit behind the requested stages");
+    static_assert(GENERAL || LA * TILEB + NW * 32 * ROWB <= STAGES * TILEB, "the epilogue's row blocks do not fit behind the requested stages");
+    static_assert(NST <= 3 && LA * TILEB + 3 * kFaithfulRows * D * 2 + 2 * 4096 + 128 <= STAGES * TILEB, "first-rows path does not fit behind the requested stages");
+    static_assert(NSTV == NST || (NSTV == NST - 1 && NSTV >= 2), "V stages: as many as K stages, or one fewer");
     constexpr uint32_t LDS_V = NST * TILEB;       // K stages first, then V stages
     static_assert(INSTR % NW == 0, "tile must divide over the waves");
-    static_assert(NST >= 2 && NST <= 4 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
+    static_assert(NST >= 2 && NST * TILEB <= 65536, "stage offsets must fit the 16-bit LDS immediate");
     typedef Num<BF16> N;
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -447,7 +454,7 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     }
     // next_slot broadcasts the list position a queue-scheduled workgroup has taken
     volatile __attribute__((address_space(3))) unsigned *next_slot =
-        (volatile __attribute__((address_space(3))) unsigned *)(uintptr_t)(lds0 + 2 * NST * TILEB);
+        (volatile __attribute__((address_space(3))) unsigned *)(uintptr_t)(lds0 + STAGES * TILEB - 64);
     constexpr unsigned kNoTicket = 0xffffffffu;
     // The work item of pass `pass_no` of this workgroup, or -1 when its work is done (list positions fit 31
     // bits, the host checks that).  Queue schedule: `ticket` is the value of the own XCD's counter when thread 0
@@ -816,9 +823,11 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     };
 
     // ---- the steady-state iteration: PV(tile-1) from V stage VST, softmax(tile), QK(tile+1) from K stage KST
-    auto steady = [&](auto KST, auto VST, int tile) __attribute__((always_inline)) {
+    auto steady = [&](auto KST, auto VST, int vstage_rt, int tile) __attribute__((always_inline)) {
         constexpr uint32_t ks = decltype(KST)::value * TILEB;
-        constexpr uint32_t vs = decltype(VST)::value * TILEB;
+        // (with as many V stages as K stages the V stage is a compile-time value like the K stage; with one fewer
+        // the two cycle with different periods, and the V stage is a run-time offset added to the lanes' addresses)
+        const uint32_t vs = NSTV == NST ? decltype(VST)::value * TILEB : (uint32_t)vstage_rt * TILEB;
         u32x4 fr[NF];                              // operand fragments, in the order they are consumed
         auto fetch = [&](int n) __attribute__((always_inline)) {
             if (n < NPV) fr[n] = read_v(vs, n);
@@ -911,13 +920,11 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
 
     unsigned ticket_ahead = kNoTicket;      // thread 0 only
     if (any_tile) {             // (GENERAL: a split, or a block of rows that sees no key, may have no tile at all)
-    // ---- prologue: K(t0) .. K(t0+LA-1) and V(t0) .. V(t0+LA-3) requested before the first iteration (iteration
-    // i requests K(i+1+LA) and V(i-1+LA), and the first one is i = t0 - 1)
+    // ---- prologue: K(t0) .. K(t0+LA-1) requested before the first iteration (iteration i requests K(i+1+LA) and
+    // V(i-1+LAV), and the first one is i = t0 - 1)
     if (!next_requested) {
         issue_k(t0, 0);
         if (LA > 1 && t0 + 1 <= t1) issue_k(t0 + 1, 1);
-        if (LA > 2 && t0 + 2 <= t1) issue_k(t0 + 2, 2);
-        if (LA > 2) issue_v(t0, 0);
     }
     next_requested = false;
     wait_vm<0>();
@@ -927,17 +934,19 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
     phase_barrier();
 
-    // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST
-    // of its tensor, so the iteration reads K stage j % NST and V stage (j - 2) % NST; it issues the loads of
-    // K(i+1+LA) and V(i-1+LA), which overwrite tiles whose last readers ran one iteration ago.
+    // Iteration j (tile i = t0 - 1 + j) does PV(i-1), softmax(i), QK(i+1).  Tile t0 + r lives in stage r % NST of
+    // K and r % NSTV of V, so the iteration reads K stage j % NST and V stage (j - 2) % NSTV; it issues the loads of
+    // K(i+1+LA) and V(i-1+LAV), which overwrite tiles whose last readers ran one iteration ago.
     // Every wave executes every iteration (one barrier each); a wave whose own tile range does not cover all
     // three pieces runs the plain pieces it has, the others run the interleaved body.  The two kinds live in
     // separate loops: merging them under one branch makes the register allocator spill.
-    auto finish_iteration = [&](bool full_issue, bool past_last_request) __attribute__((always_inline)) {
-        // What the next iteration reads must have landed: that was requested LA - 1 iterations ago, so the
-        // requests of the LA - 1 most recent iterations may stay in flight (vmcnt counts requests, so this only
-        // holds while every one of those iterations made all of its 2 * IPW requests)
-        if (NST >= 3 && full_issue) wait_vm<2 * IPW>();
+    auto finish_iteration = [&](bool more_k, bool more_v, bool past_last_request) __attribute__((always_inline)) {
+        // What the next iteration reads must have landed.  With LA = LAV = 2 that was requested one iteration ago,
+        // so this iteration's requests may stay in flight (vmcnt counts requests, so this only holds while the
+        // iteration made all of its 2 * IPW requests).  With LAV = 1 (one V stage fewer) the next iteration reads
+        // the V tile requested in this one: V is requested in front of K, and only K's requests stay in flight.
+        if (NSTV == NST && NST >= 3 && more_k && more_v) wait_vm<2 * IPW>();
+        else if (NSTV < NST && more_k) wait_vm<IPW>();
         // (the last iterations of an item, those past the request for V(t1), request nothing, and the one before
         // them has waited for everything: they do not wait, so that the counter fetched there for the next
         // item stays in flight)
@@ -978,59 +987,71 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
 #else
 #define FA_RING_CHECK(i, ks, vs, salt) do { } while (0)
 #endif
-    auto generic_iteration = [&](int i, int j3) __attribute__((always_inline)) {
-        const int tk = i + 1 + LA, tv = i - 1 + LA;
+    // V stage read by the iteration with K stage j3 and run-time V counter jv (= (j - 2) mod NSTV), and the V stage
+    // it requests into (the one read one iteration ago)
+    auto generic_iteration = [&](int i, int j3, int jv) __attribute__((always_inline)) {
+        const int tk = i + 1 + LA, tv = i - 1 + LAV;
         const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
         const int jm1 = j3 == 0 ? NST - 1 : j3 - 1, jm2 = jm1 == 0 ? NST - 1 : jm1 - 1, jm3 = jm2 == 0 ? NST - 1 : jm2 - 1;
+        const int v_read = NSTV == NST ? jm2 : jv, v_fill = NSTV == NST ? jm3 : (jv == 0 ? NSTV - 1 : jv - 1);
+        if (NSTV < NST && more_v) issue_v(tv, v_fill);     // (in front of K: see finish_iteration)
         if (more_k) issue_k(tk, jm1);              // (j + LA) % NST == (j - 1) % NST
-        if (more_v) issue_v(tv, jm3);              // (j - 2 + LA) % NST == (j - 3) % NST
-        FA_RING_CHECK(i, j3, jm2, 0);
-        if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(jm2);
+        if (NSTV == NST && more_v) issue_v(tv, v_fill);    // (j - 2 + LAV) % NSTV == (j - 3) % NSTV
+        FA_RING_CHECK(i, j3, v_read, 0);
+        if (my_lo <= i - 1 && i - 1 <= my_hi) pv_plain(v_read);
         if (my_lo <= i && i <= my_hi) softmax_plain(i);
         if (my_lo <= i + 1 && i + 1 <= my_hi) qk_plain(j3, i + 1);
-        FA_RING_CHECK(i, j3, jm2, 3);
-        finish_iteration(more_k && more_v, tv > t1);
+        FA_RING_CHECK(i, j3, v_read, 3);
+        finish_iteration(more_k, more_v, tv > t1);
     };
-    auto steady_iteration = [&](auto J3, int i) __attribute__((always_inline)) {
+    auto steady_iteration = [&](auto J3, int i, int jv) __attribute__((always_inline)) {
         constexpr int j3 = decltype(J3)::value;
         constexpr int jm1 = (j3 + NST - 1) % NST, jm2 = (j3 + 2 * NST - 2) % NST, jm3 = (j3 + 3 * NST - 3) % NST;
-        const int tk = i + 1 + LA, tv = i - 1 + LA;
+        const int tk = i + 1 + LA, tv = i - 1 + LAV;
         const bool more_k = tk <= t1, more_v = tv >= t0 && tv <= t1;
+        const int v_read = NSTV == NST ? jm2 : jv, v_fill = NSTV == NST ? jm3 : (jv == 0 ? NSTV - 1 : jv - 1);
+        if (NSTV < NST && more_v) issue_v(tv, v_fill);
 #ifdef FA_CHECK_RING_BREAK
         // the checker's negative control: the K tile goes into the stage that is being read in this iteration
         if (more_k) issue_k(tk, j3);
 #else
         if (more_k) issue_k(tk, jm1);
 #endif
-        if (more_v) issue_v(tv, jm3);
-        FA_RING_CHECK(i, j3, jm2, 1);
-        steady(IntC<j3>{}, IntC<jm2>{}, i);
-        FA_RING_CHECK(i, j3, jm2, 5);
-        finish_iteration(more_k && more_v, false);
+        if (NSTV == NST && more_v) issue_v(tv, v_fill);
+        FA_RING_CHECK(i, j3, v_read, 1);
+        steady(IntC<j3>{}, IntC<jm2>{}, v_read, i);
+        FA_RING_CHECK(i, j3, v_read, 5);
+        finish_iteration(more_k, more_v, false);
     };
-    int i = t0 - 1, j3 = 0;
+    // jv: the V stage the iteration reads, (j - 2) mod NSTV, kept as a run-time counter (used when NSTV != NST)
+    int i = t0 - 1, j3 = 0, jv = (2 * NSTV - 2) % NSTV;
+    auto advance = [&]() __attribute__((always_inline)) {
+        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+        jv = jv == NSTV - 1 ? 0 : jv + 1;
+    };
     for (; i < t1; ++i) {                 // fill: until NST consecutive iterations are steady and the stage is 0
         if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
-        generic_iteration(i, j3);
-        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+        generic_iteration(i, j3, jv);
+        advance();
     }
     for (; i >= my_lo + 1 && i + NST - 1 <= my_hi - 1 && i <= t1 + 1; i += NST) {
-        steady_iteration(IntC<0>{}, i);
-        steady_iteration(IntC<1>{}, i + 1);
-        if (NST >= 3) steady_iteration(IntC<2 % NST>{}, i + 2);
-        if (NST >= 4) steady_iteration(IntC<3 % NST>{}, i + 3);
+        steady_iteration(IntC<0>{}, i, jv);
+        advance();
+        steady_iteration(IntC<1>{}, i + 1, jv);
+        advance();
+        if (NST >= 3) { steady_iteration(IntC<2 % NST>{}, i + 2, jv); advance(); }
     }
     for (; i < t1; ++i) {                 // drain, up to the last two iterations
-        generic_iteration(i, j3);
-        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+        generic_iteration(i, j3, jv);
+        advance();
     }
     // Queue schedule: the counter round trip for the NEXT item (2.3 us) runs behind the last two iterations.
     // (Between two loops on purpose: as a branch inside generic_iteration the same statement costs the whole
     // kernel fifty registers.)
     if (a.queue != nullptr && tid == 0) ticket_ahead = atomicAdd(&a.queue[xcd], 1u);
-    for (; i <= t1 + 1; ++i) {            // the last two iterations (three stages: they request nothing any more)
-        generic_iteration(i, j3);
-        j3 = j3 == NST - 1 ? 0 : j3 + 1;
+    for (; i <= t1 + 1; ++i) {            // the last two iterations (three stages each: they request nothing any more)
+        generic_iteration(i, j3, jv);
+        advance();
     }
 
     }   // any_tile
@@ -1074,8 +1095,6 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         // (every LDS stage is free: the last iteration ended with a barrier)
         issue_k_from(nK, nt0, 0);
         if (LA > 1 && nt0 + 1 <= nt1) issue_k_from(nK, nt0 + 1, 1);
-        if (LA > 2 && nt0 + 2 <= nt1) issue_k_from(nK, nt0 + 2, 2);
-        if (LA > 2) issue_v_from(nV, nt0, 0);
         // (S is a multiple of 128: a wave has all its rows or none; one without rows never uses its fragments and
         // reads those of the block's first wave, so that no select has to wait for the data)
         const int nrow = nq0 + (nq0 + wave * WR < S ? wave * WR : 0) + l32;
@@ -1218,12 +1237,12 @@ __global__ void __launch_bounds__(256) fa_combine_splits(const FaKernelArgs a)
     if (a.lse != nullptr && c4 == 0) a.lse[row] = mx == -INFINITY ? -INFINITY : mx + __logf(wsum);
 }
 
-template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false>
+template <bool BF16, int D, bool MASKED, bool ALIBI, bool GENERAL, bool DROPOUT, int NW, int NST, bool STRIDED = false, int NSTV = NST>
 hipError_t launch(const FaKernelArgs &a, unsigned grid, hipStream_t stream, bool configure_only)
 {
     constexpr int TILEB = kBlockKeys * D * 2;
-    const size_t smem = 2 * NST * TILEB + 64;      // the stages plus the two words of the queue schedule
-    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, NST, STRIDED>;
+    const size_t smem = (NST + NSTV) * TILEB;      // the stages (the queue schedule's word borrows the last bytes between items)
+    auto kern = fa_fwd_pipelined<BF16, D, MASKED, ALIBI, GENERAL, DROPOUT, NW, NST, STRIDED, NSTV>;
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
     const unsigned long long dev_bit = 1ull << fa_launch_device();
@@ -1251,7 +1270,7 @@ hipError_t launch_forward(const FaKernelArgs &a, int bf16, int D, int masked, in
 #define FA_CASE(BF, DD, MK, AL) \
     if (bf16 == BF && D == DD && masked == MK && alibi == AL) { \
         if (shape == 0) return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 8, (GENERAL ? 2 : 3), STRIDED>(a, grid, stream, configure_only); \
-        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, 2, STRIDED>(a, grid, stream, configure_only); \
+        return launch<BF != 0, DD, MK != 0, AL != 0, GENERAL, DROPOUT, 4, (GENERAL ? 2 : FA_S1K), STRIDED, (GENERAL ? 2 : FA_S1V)>(a, grid, stream, configure_only); \
     }
 #define FA_CASES(BF, DD) FA_CASE(BF, DD, 0, 0) FA_CASE(BF, DD, 1, 0) FA_CASE(BF, DD, 0, 1) FA_CASE(BF, DD, 1, 1)
     FA_CASES(0, 64) FA_CASES(0, 128) FA_CASES(1, 64) FA_CASES(1, 128)
