@@ -381,7 +381,14 @@ def main():
             want = int((args.cpu_seconds - t1 - dt - fixed) / per_row)
             if want > 2 * n2:
                 n = min(total, want)
+                spent = t1 + dt
                 sample, dt = timed_rows(n)
+                # (the small samples run on cold caches and overestimate the cost per row: when the sized sample
+                # left more than its own time of the target unused, one more is sized from its rate)
+                left = args.cpu_seconds - spent - dt
+                if n < total and left > dt:
+                    n = min(total, int(left / (dt / n)))
+                    sample, dt = timed_rows(n)
         pairs = 0
         for r in sample.tolist():
             i = r % S

@@ -1029,18 +1029,27 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
         j3 = j3 == NST - 1 ? 0 : j3 + 1;
         jv = jv == NSTV - 1 ? 0 : jv + 1;
     };
-    for (; i < t1; ++i) {                 // fill: until NST consecutive iterations are steady and the stage is 0
-        if (j3 == 0 && i >= my_lo + 1 && i + NST - 1 <= my_hi - 1) break;
+    // An iteration in which this wave has all three pieces runs the interleaved body, whatever stage the ring is
+    // at: single iterations in front of and behind the loop over whole turns of the ring bring the stage to 0 and
+    // take what is left over (as plain pieces these iterations cost short problems 1-3 %).  Straight-line copies
+    // on purpose: one loop that picks the body by the stage makes the register allocator spill 330-520 bytes.
+    auto whole = [&](int it) __attribute__((always_inline)) { return it >= my_lo + 1 && it + 1 <= my_hi; };
+    for (; i < t1; ++i) {                 // fill: until this wave has all three pieces of an iteration
+        if (whole(i)) break;
         generic_iteration(i, j3, jv);
         advance();
     }
-    for (; i >= my_lo + 1 && i + NST - 1 <= my_hi - 1 && i <= t1 + 1; i += NST) {
+    if (j3 == 1 && whole(i)) { steady_iteration(IntC<1>{}, i, jv); advance(); ++i; }
+    if (NST >= 3 && j3 == 2 && whole(i)) { steady_iteration(IntC<2 % NST>{}, i, jv); advance(); ++i; }
+    for (; j3 == 0 && whole(i) && whole(i + NST - 1); i += NST) {
         steady_iteration(IntC<0>{}, i, jv);
         advance();
         steady_iteration(IntC<1>{}, i + 1, jv);
         advance();
         if (NST >= 3) { steady_iteration(IntC<2 % NST>{}, i + 2, jv); advance(); }
     }
+    if (j3 == 0 && whole(i)) { steady_iteration(IntC<0>{}, i, jv); advance(); ++i; }
+    if (NST >= 3 && j3 == 1 && whole(i)) { steady_iteration(IntC<1>{}, i, jv); advance(); ++i; }
     for (; i < t1; ++i) {                 // drain, up to the last two iterations
         generic_iteration(i, j3, jv);
         advance();
