@@ -136,10 +136,10 @@ def lib():
         L.fa_fwd_suggest_splits.argtypes = [ctypes.POINTER(FaFwdParams)]
         L.run_flash_attention.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
-        L.fa_sched_block_rows.argtypes = [ctypes.c_int] * 4
+        L.fa_sched_block_rows.argtypes = [ctypes.c_int] * 7
         L.fa_sched_block_keys.argtypes = [ctypes.c_int]
         L.fa_sched_num_items.restype = ctypes.c_longlong
-        L.fa_sched_num_items.argtypes = [ctypes.c_int] * 4
+        L.fa_sched_num_items.argtypes = [ctypes.c_int] * 7
         L.fa_sched_item.argtypes = [ctypes.c_int] * 7 + [ctypes.c_longlong, ctypes.POINTER(ctypes.c_int),
                                                          ctypes.POINTER(ctypes.c_int)]
         L.fa_sched_heads.argtypes = [ctypes.c_int] * 3 + [ctypes.POINTER(ctypes.c_int)] * 3

@@ -56,19 +56,36 @@ constexpr int kComputeUnits = 256;      // MI355X; the persistent grid is sized 
 // Workgroup shape for a problem.  The 8-wave kernel (256 query rows, one workgroup per CU) shares every K/V
 // tile among more rows; the 4-wave kernel (128 rows, two workgroups per CU, each with its own barrier, so that the
 // two waves of a SIMD are never lined up by one) has twice as many, smaller work items.  It wins when there are
-// too few of the large items to fill and balance the chip, and when the items are short: at S <= 1024 (ten tiles
-// per 256-row item under a causal mask), and at head dimension 64 up to S = 2048, where a tile carries half the
-// matrix work per barrier.  Measured, causal fp16, 4 waves against 8, TFLOP/s in one process: B8 H32 S1024 D64 504
-// against 432, B8 H16 S1024 D64 443 against 391, B16 H16 S512 D64 275 against 252, B8 H32 S1024 D128 653 against
-// 590, B16 H16 S512 D128 369 against 340, c2 (B4 H16 S2048 D64) 572-580 against 549-563, B4 H32 S2048 D64 638 against
-// 626; without a mask B8 H32 S1024 D64 734 against 718; and the other way round B4 H16 S2048 D128 772 against 793,
-// B2 H32 S4096 D128 907 against 958, B1 H32 S8192 D64 796 against 818, c4 783-808 against 795-796, c3 978-1002
-// against 1031-1051.
-int waves_for(int B, int N, int S, int d)
+// too few of the large items to fill and balance the chip, and when the items are short, i.e. when no query sees
+// more than 1024 keys (2048 at head dimension 64, where a tile carries half the matrix work per barrier): short
+// sequences, and windows on long ones.  Measured, causal fp16, 4 waves against 8, TFLOP/s in one process: B8 H32
+// S1024 D64 504 against 432, B8 H16 S1024 D64 443 against 391, B16 H16 S512 D64 275 against 252, B8 H32 S1024 D128 653
+// against 590, B16 H16 S512 D128 369 against 340, c2 (B4 H16 S2048 D64) 568-580 against 541-563, B4 H32 S2048 D64 638
+// against 626; windows: 512 keys at B1 H32 S16384 D128 604 against 546, 1024 keys at B2 H32 S8192 D64 618 against 578,
+// 256 keys at B4 H32 S2048 D64 275 against 241; without a mask B8 H32 S1024 D64 734 against 718; and the other way
+// round a window of 2048 keys at B1 H32 S16384 D128 867 against 899, B2 H32 S4096 D128 907 against 958, B1 H32 S8192
+// D64 796 against 818, c3 973-1002 against 1029-1051; level: c4 (window 1024, D128, which stays with 8 waves) 780
+// against 782, B2 H32 S4096 D64 731 against 732.
+// (`keys`: the largest number of keys a query can see, the key length without a mask)
+int waves_for(int B, int N, int S, int d, long long keys)
 {
-    if (S <= 1024 || (d == 64 && S <= 2048)) return 4;
+    if (S < 256) return 4;              // (few queries per head, e.g. decoding: a 256-row block would be mostly empty)
+    if (keys <= (d == 64 ? 2048 : 1024)) return 4;
     const long long big_items = (long long)B * N * ((S + 255) / 256);
     return big_items >= 2LL * kComputeUnits ? 8 : 4;
+}
+// the same from the mask as the boundary states it
+int waves_for_mask(int B, int N, int S, int S_kv, int d, int is_causal, int window_left, int window_right)
+{
+    const int sk = S_kv > 0 ? S_kv : S, s_max = sk > S ? sk : S;
+    int L, R;
+    fa_mask_bounds(s_max, is_causal, window_left, window_right, &L, &R);
+    const long long keys = (long long)L + R + 1;
+    return waves_for(B, N, S, d, keys < sk ? keys : sk);
+}
+int waves_of(const fa_fwd_params *p)
+{
+    return waves_for_mask(p->B, p->N, p->S, p->S_kv, p->d, p->is_causal, p->window_size_left, p->window_size_right);
 }
 
 thread_local char g_last_error[256] = "";
@@ -163,12 +180,15 @@ const char *fa_strerror(int status)
 
 const char *fa_last_device_error(void) { return g_last_error; }
 
-int fa_sched_block_rows(int B, int N, int S, int d) { return 32 * waves_for(B, N, S, d); }
+int fa_sched_block_rows(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
+{
+    return 32 * waves_for_mask(B, N, S, S, d, is_causal, window_left, window_right);
+}
 int fa_sched_block_keys(int d) { (void)d; return kBlockKeysHost; }
 
-long long fa_sched_num_items(int B, int N, int S, int d)
+long long fa_sched_num_items(int B, int N, int S, int d, int is_causal, int window_left, int window_right)
 {
-    const int br = fa_sched_block_rows(B, N, S, d);
+    const int br = fa_sched_block_rows(B, N, S, d, is_causal, window_left, window_right);
     return (long long)B * N * ((S + br - 1) / br);
 }
 
@@ -176,7 +196,7 @@ int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left, in
                   long long item, int *bh, int *q_begin)
 {
     if (B <= 0 || N <= 0 || S <= 0 || !bh || !q_begin) return FA_ERR_BAD_SHAPE;
-    const int br = fa_sched_block_rows(B, N, S, d);
+    const int br = fa_sched_block_rows(B, N, S, d, is_causal, window_left, window_right);
     const int nqb = (S + br - 1) / br;
     if (item < 0 || item >= (long long)B * N * nqb) return FA_ERR_BAD_SHAPE;
     int L, R, qb;
@@ -266,7 +286,7 @@ int packed_group(const fa_fwd_params *p)
     if (hk <= 0 || hk >= p->N || p->N % hk != 0) return 1;
     const int group = p->N / hk, sk = p->S_kv > 0 ? p->S_kv : p->S;
     if (sk <= p->S) return 1;                                  // queries must sit behind earlier keys
-    if ((long long)group * p->S > 32LL * waves_for(p->B, p->N, p->S, p->d)) return 1;
+    if ((long long)group * p->S > 32LL * waves_of(p)) return 1;
     return group;
 }
 // work items before key splits
@@ -274,7 +294,7 @@ long long base_items(const fa_fwd_params *p)
 {
     const int pack = packed_group(p);
     if (pack > 1) return (long long)p->B * (p->N / pack);
-    return fa_sched_num_items(p->B, p->N, p->S, p->d);
+    return fa_sched_num_items(p->B, p->N, p->S, p->d, p->is_causal, p->window_size_left, p->window_size_right);
 }
 int effective_splits(const fa_fwd_params *p)
 {
@@ -300,7 +320,7 @@ int fa_fwd_suggest_splits(const fa_fwd_params *p)
     // filling it twice: 98 against 106 us on B16 H32/8 S1 S_kv8192, 53 against 61 us on B8 H32/8 S4 S_kv8192,
     // 370 against 361 us on B4 H32 S1 S_kv32768), with at least four key tiles (256 keys) per split
     const long long items = base_items(p);
-    const long long resident = (long long)kComputeUnits * (waves_for(p->B, p->N, p->S, p->d) == 8 ? 1 : 2);
+    const long long resident = (long long)kComputeUnits * (waves_of(p) == 8 ? 1 : 2);
     if (items >= resident) return 1;
     long long n = (resident + items - 1) / items;
     const long long cap = key_tiles(p) / 4;
@@ -320,7 +340,7 @@ int validate_no_workspace(const fa_fwd_params *p)
     if (!(p->dropout_prob >= 0.0f) || !(p->dropout_prob < 1.0f)) return FA_ERR_UNSUPPORTED;
     if (!(p->softmax_scale > 0.0f) || !isfinite(p->softmax_scale)) return FA_ERR_SCALE;
     const long long bh = (long long)p->B * p->N;
-    if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
+    if (bh > 0x7fffffffLL || fa_sched_num_items(p->B, p->N, p->S, p->d, p->is_causal, p->window_size_left, p->window_size_right) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
     if (p->S_kv < 0) return FA_ERR_BAD_SHAPE;
     if ((long long)p->S + (p->S_kv > 0 ? p->S_kv : p->S) > 0x3fffffffLL) return FA_ERR_TOO_LARGE;   // tile and mask arithmetic is 32-bit
     if (base_items(p) * effective_splits(p) > 0x7fffffffLL) return FA_ERR_TOO_LARGE;
@@ -400,7 +420,7 @@ int forward(const fa_fwd_params *p, void *workspace, const FaDeviceState *ds, vo
         a.v_bs = eff[2][0]; a.v_hs = eff[2][1]; a.v_rs = (int)eff[2][2];
         a.o_bs = eff[3][0]; a.o_hs = eff[3][1]; a.o_rs = (int)eff[3][2];
     }
-    const int waves = waves_for(p->B, p->N, p->S, p->d);
+    const int waves = waves_of(p);
     const int block_rows = 32 * waves;
     a.n_qblocks = a.pack > 1 ? 1 : (p->S + block_rows - 1) / block_rows;
     const int s_max = a.Sk > p->S ? a.Sk : p->S;        // stands in for "unbounded"

@@ -216,11 +216,12 @@ const char *fa_last_device_error(void);
 /* ------------------------------------------------------------------ */
 enum { FA_TILE_SKIP = 0, FA_TILE_PARTIAL = 1, FA_TILE_FULL = 2 };
 
-/* Query rows per work item for a problem, and keys per tile for head dim d. */
-int fa_sched_block_rows(int B, int N, int S, int d);
+/* Query rows per work item for a problem (128 or 256: it depends on how many keys a query can see, so the mask
+ * is part of the question), and keys per tile for head dim d. */
+int fa_sched_block_rows(int B, int N, int S, int d, int is_causal, int window_left, int window_right);
 int fa_sched_block_keys(int d);
 /* Number of work items for a problem: B*N*ceil(S/block_rows). */
-long long fa_sched_num_items(int B, int N, int S, int d);
+long long fa_sched_num_items(int B, int N, int S, int d, int is_causal, int window_left, int window_right);
 /* Work item `item` (0 = launched first) -> batch*N+head and first query row. */
 int fa_sched_item(int B, int N, int S, int d, int is_causal, int window_left,
                   int window_right, long long item, int *bh, int *q_begin);

@@ -76,8 +76,8 @@ def test_tile_range_equals_reference_formulas(fa):
 def test_every_item_once_and_longest_first(fa, shape, causal, wl, wr):
     L = fa.lib()
     B, N, S, d = shape
-    n = L.fa_sched_num_items(B, N, S, d)
-    br, bk = L.fa_sched_block_rows(B, N, S, d), L.fa_sched_block_keys(d)
+    n = L.fa_sched_num_items(B, N, S, d, causal, wl, wr)
+    br, bk = L.fa_sched_block_rows(B, N, S, d, causal, wl, wr), L.fa_sched_block_keys(d)
     assert br in (128, 256)
     assert n == B * N * ((S + br - 1) // br)
     seen = set()
