@@ -322,13 +322,14 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
 
 
 def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                             alibi_slopes=None, dropout_prob=0.0, seed=0, five_products="auto"):
+                             alibi_slopes=None, dropout_prob=0.0, seed=0, five_products="auto", poison_workspace=False):
     """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
     fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask, slopes, dropout
     probability and seed.
     ``five_products``: True asks for the workspace that selects the five-product form (fa_bwd_fast_workspace_bytes:
     B*N*S*S elements more), False for the small one; "auto" takes the large one when the problem qualifies and it
-    is at most a quarter of the device's free memory.
+    is at most a quarter of the device's free memory.  ``poison_workspace`` (for tests) fills the workspace with
+    NaN bit patterns first: the kernels must not read anything in it that they have not written.
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
     import torch
@@ -370,6 +371,8 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     if fast and (five_products is True or fast <= _ws_budget(q.device)):
         need = fast
     workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)     # stream-ordered: freed after the launch
+    if poison_workspace:
+        workspace.fill_(0xff)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), need
     st = lib().fa_bwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream))
     if st != FA_OK:

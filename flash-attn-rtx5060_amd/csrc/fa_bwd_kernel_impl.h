@@ -381,13 +381,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
 // LDS stage: Q (row-wise for S = Q K^T, transposed for dK^T += Q^T dS), dO (row-wise for dP = dO V^T, transposed
 // for dV^T += dO^T P), 64 rescaled logsumexps, 64 deltas.
 // ---------------------------------------------------------------------------------------------------------
-// WRITE_DS (reference layout only): every 32-query x 32-key block of dS that a wave forms is also written to
+// WRITE_DS (regular lengths, no ALiBi, no dropout): every 32-query x 32-key block of dS that a wave forms is also written to
 // a.ds_blocks, in the wave's operand order, for fa_bwd_dq_from_ds.
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, bool WRITE_DS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
     constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
-    static_assert(!WRITE_DS || LAYOUT == 0, "dS blocks are written for the reference's layout only");
+    static_assert(!WRITE_DS || (LAYOUT <= 1 && !ALIBI && !DROPOUT), "dS blocks are written for regular lengths without ALiBi and dropout only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
@@ -600,7 +600,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             // Block (32-query block 2t + qb, this wave's 32-key block) of dS, 2 KiB, as the registers hold it: this
             // lane's key against the queries 8g + 4*half + 0..3, g = 0..3.  Two store instructions of 1 KiB each,
             // lane l writing bytes 16 l .. 16 l + 15 of its KiB: queries of g = 0, 1 in the first, g = 2, 3 in the second.
-            const long long block = (long long)bhk * fa_ds_blocks_per_head(S) + fa_ds_block_index(S, 2 * t + qb, kw >> 5);
+            // (bhq: the QUERY head, batch * H + head; the blocks of the query heads that share this K/V head are apart)
+            const long long block = (long long)bhq * fa_ds_blocks_per_head(S) + fa_ds_block_index(S, 2 * t + qb, kw >> 5);
             // (Inline assembly: the block's address stays in two scalar registers and the lane's offset in one
             // vector register that lives for these two instructions only -- as a 64-bit vector address it cost
             // the registers that made the compiler spill inside the tile loop, and every reload from scratch
@@ -722,7 +723,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// The five-product form (reference layout only).  fa_bwd_dq above and fa_bwd_dkdv each recompute S and dP: seven
+// The five-product form (regular lengths in the reference's or a strided layout, no ALiBi, no dropout).  fa_bwd_dq above and fa_bwd_dkdv each recompute S and dP: seven
 // products for five.  Here fa_bwd_dkdv, which has every dS block in registers as the operand of dK += dS^T Q,
 // also writes it out (WRITE_DS), and dQ = scale * dS K is one product over those blocks: every output element
 // still has exactly one writer and the same inputs give the same bits.  The price is S*S_kv storage-type elements
@@ -731,7 +732,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
 // fa_bwd_prepare: delta_i = sum_t dO_it O_it and the logsumexp in exp2 units, which fa_bwd_dkdv fetches per
 // query tile (fa_bwd_dq writes them in the seven-product form).
 // ---------------------------------------------------------------------------------------------------------
-template <bool BF16, int D>
+template <bool BF16, int D, bool STRIDED>
 __global__ void __launch_bounds__(256) fa_bwd_prepare(const FaBwdArgs a)
 {
     constexpr int TPR = D / 8;                    // threads per row, 16 bytes each
@@ -740,8 +741,15 @@ __global__ void __launch_bounds__(256) fa_bwd_prepare(const FaBwdArgs a)
     const bool live = row < n_rows;
     const long long r = live ? row : n_rows - 1;
     const int c = (threadIdx.x % TPR) * 8;
-    const u32x4 o = *reinterpret_cast<const u32x4 *>(a.O + r * D + c);
-    const u32x4 g = *reinterpret_cast<const u32x4 *>(a.dO + r * D + c);
+    const uint16_t *o_row = a.O + r * D, *g_row = a.dO + r * D;
+    if (STRIDED) {                                // row r of the [B,H,S] order, wherever the tensors keep it
+        const long long bh = r / a.S;
+        const int i = (int)(r - bh * a.S), b = (int)(bh / a.H), h = (int)(bh - (long long)b * a.H);
+        o_row = head_ptr(a.O, a.o, b, h) + (long long)i * a.o.rs;
+        g_row = head_ptr(a.dO, a.dO_, b, h) + (long long)i * a.dO_.rs;
+    }
+    const u32x4 o = *reinterpret_cast<const u32x4 *>(o_row + c);
+    const u32x4 g = *reinterpret_cast<const u32x4 *>(g_row + c);
     float sum = 0.0f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -764,7 +772,7 @@ __global__ void __launch_bounds__(256) fa_bwd_prepare(const FaBwdArgs a)
 // fetched by that wave alone.  A block comes in as it lies in memory except that the 64-byte groups of four keys
 // are XOR-permuted among the four 512-byte planes, so that the transposing read of a half-wave -- four keys, all
 // 32 queries, i.e. one group in each plane -- touches every LDS bank once.
-template <bool BF16, int D, bool MASKED>
+template <bool BF16, int D, bool MASKED, bool STRIDED>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaBwdArgs a)
 {
     typedef Num<BF16> N;
@@ -790,6 +798,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     fa_item_decode(item, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
     const uint16_t *Kh = a.K + (size_t)bh * S * D;
     uint16_t *dQh = a.dQ + (size_t)bh * S * D;
+    int k_rs = D, dq_rs = D;
+    if (STRIDED) {                                 // (bh counts query heads; the K/V head of query head h is h / (H / Hk))
+        const int b = bh / a.H, h = bh - b * a.H;
+        Kh = head_ptr(a.K, a.k, b, h / (a.H / a.Hk));
+        dQh = head_ptr(a.dQ, a.dq, b, h);
+        k_rs = a.k.rs; dq_rs = a.dq.rs;
+    }
     const int q0 = qblock * 256, qw = q0 + wave * 32;
     const bool active = qw < S;                    // the last block may own fewer than 256 rows
     int t0, t1, my_lo = 1, my_hi = 0;
@@ -800,7 +815,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     const int my_qb = active ? qw >> 5 : 0;
 
     Reader rd; rd.init(lane, lds0);
-    Loader ldk; ldk.init(wave, lane, D * 2);
+    Loader ldk; ldk.init(wave, lane, k_rs * 2);
     // Source of the 16 bytes lane l brings in with instruction w (0, 1) of a block: LDS slot 64 w + l of the block
     // = plane p = 2 w + l / 32, position l % 32; that position holds key ((l % 32 / 4) ^ p) * 4 + l % 4, which lies
     // in memory at 1 KiB * w + 512 * (l / 32) + 16 * key.
@@ -825,7 +840,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     }
     auto issue = [&](int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
-        ldk.load(Kh + (size_t)tile * 64 * D, base);
+        ldk.load(Kh + (size_t)tile * 64 * k_rs, base);
         if (my_lo <= tile && tile <= my_hi) {
             const char *src = ds_head + fa_ds_block_index(S, my_qb, 2 * tile) * kDsBlockBytes;      // (and its neighbour 2 tile + 1)
             const uint32_t dst = base + TILEB + wave * WAVE_DS;
@@ -886,7 +901,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
                 u32x2 w;
                 w[0] = N::pack2(dq[db][4 * g] * a.scale, dq[db][4 * g + 1] * a.scale);
                 w[1] = N::pack2(dq[db][4 * g + 2] * a.scale, dq[db][4 * g + 3] * a.scale);
-                *reinterpret_cast<u32x2 *>(dQh + (size_t)my_q * D + 32 * db + 8 * g + 4 * half) = w;
+                *reinterpret_cast<u32x2 *>(dQh + (size_t)my_q * dq_rs + 32 * db + 8 * g + 4 * half) = w;
             }
     }
     }   // next work item
@@ -902,8 +917,9 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
     const int smem_dkdv_ds = kBwdStages * (2 * TILEB + 512) + (D == 128 ? 32 * kBwdWaves * 64 : 0);      // + the parked fragments
     auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
     auto kkv = fa_bwd_dkdv<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
-    // the five-product form: reference layout only
-    constexpr bool FIVE = LAYOUT == 0 && !ALIBI && !DROPOUT;
+    // the five-product form: regular lengths (the reference's layout or a strided one), no ALiBi, no dropout
+    constexpr bool FIVE = LAYOUT <= 1 && !ALIBI && !DROPOUT;
+    constexpr int FL = FIVE ? LAYOUT : 0;
     const int smem_dq_ds = kBwdStages * (TILEB + kBwdWaves * 2 * kDsBlockBytes);
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
     static std::atomic<unsigned long long> configured{0ull};
@@ -914,10 +930,10 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
         if (e != hipSuccess) return e;
         if constexpr (FIVE) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, 0, false, false, true>),
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, FL, false, false, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv_ds);
             if (e != hipSuccess) return e;
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED>),
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq_ds);
             if (e != hipSuccess) return e;
         }
@@ -947,9 +963,9 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
             // delta and the rescaled logsumexp; dK, dV and the dS blocks; dQ from the blocks
             constexpr int rows_per_block = 256 / (D / 8);
             const long long n_rows = (long long)a.B * a.H * a.S;
-            hipLaunchKernelGGL((fa_bwd_prepare<BF16, D>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
-            hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, 0, false, false, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
-            hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
+            hipLaunchKernelGGL((fa_bwd_prepare<BF16, D, FL == 1>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, false, false, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
+            hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
             return hipGetLastError();
         }
     }

@@ -57,20 +57,22 @@ constexpr int kComputeUnits = 256;      // MI355X; the persistent grid is sized 
 // tile among more rows; the 4-wave kernel (128 rows, two workgroups per CU, each with its own barrier, so that the
 // two waves of a SIMD are never lined up by one) has twice as many, smaller work items.  It wins when there are
 // too few of the large items to fill and balance the chip, and when the items are short, i.e. when no query sees
-// more than 1024 keys (2048 at head dimension 64, where a tile carries half the matrix work per barrier): short
-// sequences, and windows on long ones.  Measured, causal fp16, 4 waves against 8, TFLOP/s in one process: B8 H32
+// more than 1024 keys (at head dimension 64, where a tile carries half the matrix work per barrier, 4096 under a
+// mask and 2048 without one): short sequences, and windows on long ones.  Measured, causal fp16, 4 waves against 8, TFLOP/s in one process: B8 H32
 // S1024 D64 504 against 432, B8 H16 S1024 D64 443 against 391, B16 H16 S512 D64 275 against 252, B8 H32 S1024 D128 653
 // against 590, B16 H16 S512 D128 369 against 340, c2 (B4 H16 S2048 D64) 568-580 against 541-563, B4 H32 S2048 D64 638
 // against 626; windows: 512 keys at B1 H32 S16384 D128 604 against 546, 1024 keys at B2 H32 S8192 D64 618 against 578,
 // 256 keys at B4 H32 S2048 D64 275 against 241; without a mask B8 H32 S1024 D64 734 against 718; and the other way
 // round a window of 2048 keys at B1 H32 S16384 D128 867 against 899, B2 H32 S4096 D128 907 against 958, B1 H32 S8192
 // D64 796 against 818, c3 973-1002 against 1029-1051; level: c4 (window 1024, D128, which stays with 8 waves) 780
-// against 782, B2 H32 S4096 D64 731 against 732.
+// against 782.  Head dimension 64 at 4096 keys: causal B2 H32 751 against 744, B8 H32 774 against 748, B1 H16 455
+// against 443, windows of 3000 and 4096 keys at B2 H32 S8192 728 against 688 and 736 against 683; without a mask B2 H32
+// S4096 868 against 888.
 // (`keys`: the largest number of keys a query can see, the key length without a mask)
-int waves_for(int B, int N, int S, int d, long long keys)
+int waves_for(int B, int N, int S, int d, long long keys, bool masked)
 {
     if (S < 256) return 4;              // (few queries per head, e.g. decoding: a 256-row block would be mostly empty)
-    if (keys <= (d == 64 ? 2048 : 1024)) return 4;
+    if (keys <= (d == 64 ? (masked ? 4096 : 2048) : 1024)) return 4;
     const long long big_items = (long long)B * N * ((S + 255) / 256);
     return big_items >= 2LL * kComputeUnits ? 8 : 4;
 }
@@ -81,7 +83,7 @@ int waves_for_mask(int B, int N, int S, int S_kv, int d, int is_causal, int wind
     int L, R;
     fa_mask_bounds(s_max, is_causal, window_left, window_right, &L, &R);
     const long long keys = (long long)L + R + 1;
-    return waves_for(B, N, S, d, keys < sk ? keys : sk);
+    return waves_for(B, N, S, d, keys < sk ? keys : sk, L < s_max || R < s_max);
 }
 int waves_of(const fa_fwd_params *p)
 {
@@ -661,22 +663,12 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
 }
 
 namespace {
-// the reference's layout and nothing else: contiguous [B,N,S,d], S a multiple of 128, as many keys and K/V heads,
-// no ALiBi, no dropout
+// what the contiguous and the strided kernels run: S a multiple of 128 and as many keys, in any storage order and
+// with any grouping of K/V heads; no ALiBi, no dropout
 bool five_product_shape(const fa_bwd_params *p)
 {
-    if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S) || (p->n_kv_heads != 0 && p->n_kv_heads != p->N)) return false;
-    if (p->alibi_slopes_ptr != nullptr || p->dropout_prob > 0.0f) return false;
-    const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
-                                   p->dq_strides, p->dk_strides, p->dv_strides};
-    const long long dense[3] = {(long long)p->N * p->S * p->d, (long long)p->S * p->d, p->d};
-    for (int t = 0; t < 8; ++t) {
-        const long long *st = strides[t];
-        if (st[0] == 0 && st[1] == 0 && st[2] == 0) continue;
-        for (int k = 0; k < 3; ++k)
-            if (st[k] != dense[k]) return false;
-    }
-    return true;
+    if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S)) return false;
+    return p->alibi_slopes_ptr == nullptr && !(fa_dropout_threshold(p->dropout_prob) != 0);
 }
 unsigned long long ds_blocks_offset(const fa_bwd_params *p)
 {

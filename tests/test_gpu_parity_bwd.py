@@ -113,15 +113,61 @@ def test_five_product_form_against_the_fp64_oracle(fa, oracle, shape, dtype, cau
         assert torch.equal(a_.view(torch.int16), b_.view(torch.int16))
 
 
-def test_five_product_workspace_is_offered_for_the_reference_layout_only(fa):
+def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
+    """Lengths a multiple of 128 with as many keys, in any storage order and with any grouping of K/V heads (the dS
+    blocks are per QUERY head); not with other lengths, ALiBi or dropout."""
     import ctypes
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128)
     small = L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok)))
-    assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == ((small + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
-    for other in (dict(S=1000), dict(S_kv=2048), dict(n_kv_heads=2), dict(dropout_prob=0.1), dict(alibi_ptr=256),
-                  dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)})):
+    large = ((small + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
+    assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == large
+    for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)})):
+        assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **same}))) == large, same
+    for other in (dict(S=1000), dict(S_kv=2048), dict(dropout_prob=0.1), dict(alibi_ptr=256)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
+
+
+FIVE_STRIDED = [
+    # B, H, Hk, S, D, dtype, causal, wl, wr, bshd: regular lengths through the strided kernels
+    (2, 4, 2, 512, 128, 0, True, -1, -1, True),
+    (1, 4, 4, 384, 64, 1, True, 100, -1, True),
+    (1, 6, 2, 256, 64, 0, False, -1, -1, False),
+    (1, 2, 1, 640, 128, 1, False, 64, 64, True),
+    (1, 8, 2, 768, 128, 0, True, -1, -1, True),
+    (2, 3, 1, 384, 128, 0, False, 0, 40, False),
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,D,dtype,causal,wl,wr,bshd", FIVE_STRIDED)
+def test_five_product_form_in_strided_layouts_and_with_grouped_heads(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd):
+    """The five-product form through the strided kernels ([B,S,H,D] storage, K/V heads shared by groups of query
+    heads: the key-owning workgroup writes the dS blocks of every query head of its group), against the fp64 oracle
+    and with a NaN-filled workspace, twice with the same bits; the seven-product form of the same call meets the same bars."""
+    import torch
+    q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=720 + S)
+    do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=721 + S)
+    _, k, v = make_inputs(fa, (B, Hk, S, D), dtype, seed=722 + S)
+    dq_ref, dk_ref, dv_ref = oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, None)
+    tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
+    if bshd:
+        tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
+    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, exact_first_rows=True)
+    five = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=True,
+                                       poison_workspace=True)
+    seven = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=False)
+    again = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=True,
+                                        poison_workspace=True)
+    torch.cuda.synchronize()
+    for name, got, want, other, rerun, like in zip(("dQ", "dK", "dV"), five, (dq_ref, dk_ref, dv_ref), seven, again, (tq, tk, tv)):
+        assert got.stride() == like.stride()
+        err = grad_errors(oracle.to_f32(from_torch(got.contiguous()), dtype), want)
+        print("five products, strided", (B, H, Hk, S, D), dtype, causal, wl, wr, bshd, name, err, flush=True)
+        check(err, dtype, name)
+        assert torch.equal(got.contiguous().view(torch.int16), rerun.contiguous().view(torch.int16)), name
+        # (the seven-product form sums delta and dQ in other orders: close, not equal)
+        close = grad_errors(oracle.to_f32(from_torch(other.contiguous()), dtype), want)
+        check(close, dtype, name + " (seven products)")
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
@@ -250,11 +296,13 @@ def test_general_layouts_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D
         check(err, dtype, name)
 
 
+@pytest.mark.parametrize("five", [False, True])
 @pytest.mark.parametrize("D,dtype,causal,wl", [(128, 0, True, -1), (64, 1, False, -1), (128, 1, True, 200), (64, 0, True, -1)])
-def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl):
+def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl, five):
     """[B,S,H,D] storage goes through the strided kernels, [B,H,S,D] through the plain ones: same values, same
-    arithmetic in the same order, so dQ, dK and dV have to agree bit for bit.  (The seven-product form, which is the
-    only one the strided layout has; the five-product form of the reference's layout sums in another order.)"""
+    arithmetic in the same order, so dQ, dK and dV have to agree bit for bit, in the seven-product form and in the
+    five-product form (which sums dQ in another order than the seven-product one, but in the same order in both
+    layouts)."""
     import torch
     B, H, S = 2, 3, 768
     q, k, v = make_inputs(fa, (B, H, S, D), dtype, seed=910 + D)
@@ -264,7 +312,7 @@ def test_storage_order_changes_no_bit_of_the_gradients(fa, D, dtype, causal, wl)
     got = []
     for tq, tk, tv, tdo in (dense, bshd):
         o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl)
-        got.append(fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, five_products=False))
+        got.append(fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, five_products=five))
     torch.cuda.synchronize()
     assert got[1][0].stride() == bshd[0].stride()
     for name, a, b in zip(("dQ", "dK", "dV"), got[0], got[1]):
