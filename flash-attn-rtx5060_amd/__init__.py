@@ -50,7 +50,8 @@ EXPORTED_SYMBOLS = (
     "fa_sched_block_rows", "fa_sched_block_keys", "fa_sched_num_items", "fa_sched_item",
     "fa_sched_heads", "fa_sched_tile_range", "fa_sched_classify", "fa_count_pairs", "fa_algorithmic_flops",
     "fa_dropout_threshold", "fa_dropout_keep", "fa_fwd_workspace_bytes", "fa_fwd_suggest_splits",
-    "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_fast_workspace_bytes", "fa_bwd_algorithmic_flops",
+    "fa_bwd_validate", "fa_bwd", "fa_bwd_workspace_bytes", "fa_bwd_fast_workspace_bytes", "fa_bwd_min_fast_workspace_bytes",
+    "fa_bwd_algorithmic_flops",
     "fa_bwd_sched_query_tile_range", "fa_bwd_sched_classify",
     "fa_dev_count", "fa_dev_name", "fa_dev_malloc", "fa_dev_free", "fa_dev_h2d", "fa_dev_d2h",
     "fa_dev_memset", "fa_dev_sync", "fa_event_create", "fa_event_record", "fa_event_sync",
@@ -157,6 +158,8 @@ def lib():
         L.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
         L.fa_bwd_fast_workspace_bytes.restype = ctypes.c_ulonglong
         L.fa_bwd_fast_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
+        L.fa_bwd_min_fast_workspace_bytes.restype = ctypes.c_ulonglong
+        L.fa_bwd_min_fast_workspace_bytes.argtypes = [ctypes.POINTER(FaBwdParams)]
         L.fa_bwd_algorithmic_flops.restype = ctypes.c_double
         L.fa_bwd_algorithmic_flops.argtypes = [ctypes.c_int] * 7
         L.fa_bwd_sched_query_tile_range.restype = None
@@ -322,13 +325,16 @@ def make_bwd_params(B, N, S, d, q_ptr=0, k_ptr=0, v_ptr=0, o_ptr=0, do_ptr=0, ls
 
 
 def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=False, window_left=-1, window_right=-1,
-                             alibi_slopes=None, dropout_prob=0.0, seed=0, five_products="auto", poison_workspace=False):
+                             alibi_slopes=None, dropout_prob=0.0, seed=0, five_products="auto", poison_workspace=False,
+                             workspace_limit=None):
     """dq, dk, dv = gradients of attention(q, k, v) given the gradient ``do`` of its output, on the GPU through
     fa_bwd().  o and lse are what flash_attention_forward returned for the same q, k, v, mask, slopes, dropout
     probability and seed.
     ``five_products``: True asks for the workspace that selects the five-product form (fa_bwd_fast_workspace_bytes:
-    B*N*S*S elements more), False for the small one; "auto" takes the large one when the problem qualifies and it
-    is at most a quarter of the device's free memory.  ``poison_workspace`` (for tests) fills the workspace with
+    B*N*S*S elements more), False for the small one; "auto" takes, when the problem qualifies, the dS blocks of about
+    2 GiB worth of heads (the form then runs over the heads in chunks, which measures no slower), at least
+    fa_bwd_min_fast_workspace_bytes and at most a quarter of the device's free memory, or ``workspace_limit`` bytes
+    when that is given; when even the least does not fit, the small one.  ``poison_workspace`` (for tests) fills the workspace with
     NaN bit patterns first: the kernels must not read anything in it that they have not written.
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
@@ -368,8 +374,25 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
                         dropout_prob=dropout_prob, seed=seed)
     need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
     fast = lib().fa_bwd_fast_workspace_bytes(ctypes.byref(p)) if five_products else 0
-    if fast and (five_products is True or fast <= _ws_budget(q.device)):
+    if fast and five_products is True and workspace_limit is None:
         need = fast
+    elif fast:
+        # "auto": whole chunks of eight K/V heads' dS blocks, about 2 GiB of them (chunks measure no slower than the
+        # full size: B2 N32 S8192 D128 3.27 ms with 2.2 or 4.4 GB against 3.34 with 8.6), never fewer heads than the
+        # library accepts and never more bytes than the limit; a size that depends on the problem alone, so that
+        # torch's allocator hands the same block back call after call
+        least = lib().fa_bwd_min_fast_workspace_bytes(ctypes.byref(p))
+        off = (need + 255) // 256 * 256
+        kv_total = q.shape[0] * k.shape[1]
+        per_head = (fast - off) // kv_total
+        heads = max((least - off) // per_head, (2 << 30) // per_head // 8 * 8)
+        limit = workspace_limit if workspace_limit is not None else _ws_budget(q.device)
+        if off + heads * per_head > limit:
+            heads = (limit - off) // per_head // 8 * 8 if limit > off else 0
+        if heads >= kv_total and fast <= limit:
+            need = fast
+        elif heads > 0 and off + heads * per_head >= least:
+            need = off + heads * per_head
     workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)     # stream-ordered: freed after the launch
     if poison_workspace:
         workspace.fill_(0xff)

@@ -24,6 +24,11 @@ struct FaBwdArgs {
     const float *alibi;                     // [H] slopes or NULL
     FaBwdTensor q, k, v, o, dO_, dq, dk, dv;
     int B, H, Hk;                           // query heads, K/V heads (Hk divides H)
+    // The K/V heads this launch works on, counted through the batch (batch * Hk + head): [head0, head0 + heads), and
+    // with them the query heads [head0 * H/Hk, (head0 + heads) * H/Hk).  All of them, except in the five-product form
+    // with a workspace that holds the dS blocks of only `ds_heads` K/V heads' groups at a time: then the key-owning
+    // and the query-owning kernel are launched once per such chunk, and block addresses count from the chunk's start.
+    int head0, heads, ds_heads;
     int S, Sk;                              // queries, keys; query i sits at key position i + Sk - S
     int L, R;                               // key j visible to the query at position p iff p - L <= j <= p + R
     float scale;

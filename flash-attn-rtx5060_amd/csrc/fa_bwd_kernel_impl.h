@@ -402,7 +402,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // one K/V head per XCD at a time; key block 0 is seen by the most queries and goes first
     // (work items as in fa_bwd_dq; the list here is ascending in the key block, which is longest first under a
     // causal mask: key block 0 is seen by every query)
-    const long long n_items = (long long)a.B * a.Hk * n_kblocks;
+    const long long n_items = (long long)a.heads * n_kblocks;
     for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (strided and general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
@@ -411,7 +411,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     if (!ONE_ITEM) asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31;
     int bhk, kblock;
-    fa_item_decode(item, a.B * a.Hk, n_kblocks, 0, &bhk, &kblock);
+    fa_item_decode(item, a.heads, n_kblocks, 0, &bhk, &kblock);
+    bhk += a.head0;
     const int b = bhk / a.Hk, hk = bhk - b * a.Hk;
     const int q_rs = STRIDES ? a.q.rs : D, g_rs = STRIDES ? a.dO_.rs : D, k_rs = STRIDES ? a.k.rs : D, v_rs = STRIDES ? a.v.rs : D;
     const uint16_t *Kh, *Vh;
@@ -601,7 +602,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             // lane's key against the queries 8g + 4*half + 0..3, g = 0..3.  Two store instructions of 1 KiB each,
             // lane l writing bytes 16 l .. 16 l + 15 of its KiB: queries of g = 0, 1 in the first, g = 2, 3 in the second.
             // (bhq: the QUERY head, batch * H + head; the blocks of the query heads that share this K/V head are apart)
-            const long long block = (long long)bhq * fa_ds_blocks_per_head(S) + fa_ds_block_index(S, 2 * t + qb, kw >> 5);
+            const long long block = (long long)(bhq - (uint32_t)(a.head0 * G)) * fa_ds_blocks_per_head(S) + fa_ds_block_index(S, 2 * t + qb, kw >> 5);
             // (Inline assembly: the block's address stays in two scalar registers and the lane's offset in one
             // vector register that lives for these two instructions only -- as a 64-bit vector address it cost
             // the registers that made the compiler spill inside the tile loop, and every reload from scratch
@@ -786,7 +787,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int S = a.S;
     const int n_qblocks = (S + 255) / 256;
-    const long long n_items = (long long)a.B * a.H * n_qblocks;
+    const int group = STRIDED ? a.H / a.Hk : 1, heads_q = a.heads * group, head0_q = a.head0 * group;
+    const long long n_items = (long long)heads_q * n_qblocks;
     for (int pass = 0;; ++pass) {
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
@@ -795,13 +797,14 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     asm volatile("" : "+v"(lane));
     const int half = lane >> 5, l32 = lane & 31, l16 = lane & 15;
     int bh, qblock;
-    fa_item_decode(item, a.B * a.H, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
+    fa_item_decode(item, heads_q, n_qblocks, MASKED ? 1 : 0, &bh, &qblock);
+    bh += head0_q;
     const uint16_t *Kh = a.K + (size_t)bh * S * D;
     uint16_t *dQh = a.dQ + (size_t)bh * S * D;
     int k_rs = D, dq_rs = D;
     if (STRIDED) {                                 // (bh counts query heads; the K/V head of query head h is h / (H / Hk))
         const int b = bh / a.H, h = bh - b * a.H;
-        Kh = head_ptr(a.K, a.k, b, h / (a.H / a.Hk));
+        Kh = head_ptr(a.K, a.k, b, h / group);
         dQh = head_ptr(a.dQ, a.dq, b, h);
         k_rs = a.k.rs; dq_rs = a.dq.rs;
     }
@@ -811,7 +814,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     fa_tile_range(S, 64, a.L, a.R, q0, S - q0 < 256 ? S - q0 : 256, &t0, &t1);
     if (active) fa_tile_range(S, 64, a.L, a.R, qw, 32, &my_lo, &my_hi);
     // this head's dS blocks; this wave reads those of query block qw / 32
-    const char *ds_head = reinterpret_cast<const char *>(a.ds_blocks) + (long long)bh * fa_ds_blocks_per_head(S) * kDsBlockBytes;
+    const char *ds_head = reinterpret_cast<const char *>(a.ds_blocks) + (long long)(bh - head0_q) * fa_ds_blocks_per_head(S) * kDsBlockBytes;
     const int my_qb = active ? qw >> 5 : 0;
 
     Reader rd; rd.init(lane, lds0);
@@ -908,11 +911,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
 }
 
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
-hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream, bool configure_only = false)
+hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stream, bool configure_only = false)
 {
     constexpr int TILEB = 64 * D * 2;
-    const unsigned grid_q = (unsigned)((long long)a.B * a.H * ((a.S + 255) / 256));
-    const unsigned grid_k = (unsigned)((long long)a.B * a.Hk * ((a.Sk + 255) / 256));
+    FaBwdArgs a = a_in;
+    const int all_heads = a.B * a.Hk, group = a.Hk > 0 ? a.H / a.Hk : 1;
+    a.head0 = 0;
+    a.heads = all_heads;
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512) + (DROPOUT ? kBwdWaves * 128 : 0);
     const int smem_dkdv_ds = kBwdStages * (2 * TILEB + 512) + (D == 128 ? 32 * kBwdWaves * 64 : 0);      // + the parked fragments
     auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
@@ -956,19 +961,31 @@ hipError_t launch_bwd(const FaBwdArgs &a, int compute_units, hipStream_t stream,
     // them their 128-wide kernels spill ten times as much, and a reload inside the tile loop waits for every tile
     // load in flight: c3's shape stored [B,S,H,D] 4.1 ms against 3.8.)
     const bool uneven = LAYOUT == 0 && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
-    const unsigned launch_q = (uneven && grid_q > resident && grid_q < 16u * resident) ? resident : grid_q;
-    const unsigned launch_k = (uneven && grid_k > resident && grid_k < 16u * resident) ? resident : grid_k;
+    auto grid_for = [&](long long items) {
+        const unsigned g = (unsigned)items;
+        return (uneven && g > resident && g < 16u * resident) ? resident : g;
+    };
     if constexpr (FIVE) {
         if (a.ds_blocks != nullptr) {
-            // delta and the rescaled logsumexp; dK, dV and the dS blocks; dQ from the blocks
+            // delta and the rescaled logsumexp, for all heads at once; then, for as many heads at a time as the
+            // workspace holds dS blocks for: dK, dV and the dS blocks; dQ from the blocks
             constexpr int rows_per_block = 256 / (D / 8);
             const long long n_rows = (long long)a.B * a.H * a.S;
             hipLaunchKernelGGL((fa_bwd_prepare<BF16, D, FL == 1>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
-            hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, false, false, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
-            hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
+            const int chunk = a.ds_heads > 0 && a.ds_heads < all_heads ? a.ds_heads : all_heads;
+            for (int h0 = 0; h0 < all_heads; h0 += chunk) {
+                a.head0 = h0;
+                a.heads = all_heads - h0 < chunk ? all_heads - h0 : chunk;
+                const unsigned launch_k = grid_for((long long)a.heads * ((a.Sk + 255) / 256));
+                const unsigned launch_q = grid_for((long long)a.heads * group * ((a.S + 255) / 256));
+                hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, false, false, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
+                hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
+            }
             return hipGetLastError();
         }
     }
+    const unsigned launch_q = grid_for((long long)a.B * a.H * ((a.S + 255) / 256));
+    const unsigned launch_k = grid_for((long long)a.B * a.Hk * ((a.Sk + 255) / 256));
     hipLaunchKernelGGL(kq, dim3(launch_q), dim3(kBwdWaves * 64), smem_dq, stream, a);
     hipLaunchKernelGGL(kkv, dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv, stream, a);
     return hipGetLastError();

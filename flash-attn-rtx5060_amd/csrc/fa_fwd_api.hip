@@ -674,7 +674,30 @@ unsigned long long ds_blocks_offset(const fa_bwd_params *p)
 {
     return (fa_bwd_workspace_bytes(p) + 255ull) & ~255ull;
 }
+// K/V heads (counted through the batch) and the bytes of dS blocks that belong to one of them: those of its group
+// of query heads
+long long kv_heads_total(const fa_bwd_params *p) { return (long long)p->B * (p->n_kv_heads > 0 ? p->n_kv_heads : p->N); }
+unsigned long long ds_bytes_per_kv_head(const fa_bwd_params *p)
+{
+    const int group = p->n_kv_heads > 0 ? p->N / p->n_kv_heads : 1;
+    return (unsigned long long)group * (unsigned long long)fa_ds_blocks_per_head(p->S) * 2048ull;
+}
+// The fewest K/V heads a chunk of the five-product form may hold: enough key blocks for two rounds of a full chip,
+// a multiple of eight (one head per XCD); all of them when the problem has no more.
+long long min_chunk_kv_heads(const fa_bwd_params *p)
+{
+    const long long key_blocks = (p->S + 255) / 256, all = kv_heads_total(p);
+    long long n = (2LL * kComputeUnits + key_blocks - 1) / key_blocks;
+    n = (n + 7) / 8 * 8;
+    return n < all ? n : all;
+}
 }  // namespace
+
+unsigned long long fa_bwd_min_fast_workspace_bytes(const fa_bwd_params *p)
+{
+    if (fa_bwd_fast_workspace_bytes(p) == 0) return 0;
+    return ds_blocks_offset(p) + (unsigned long long)min_chunk_kv_heads(p) * ds_bytes_per_kv_head(p);
+}
 
 unsigned long long fa_bwd_fast_workspace_bytes(const fa_bwd_params *p)
 {
@@ -735,9 +758,20 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.delta = static_cast<float *>(p->workspace);
     a.lse2 = a.delta + (size_t)p->B * p->N * p->S;
     // a workspace large enough for the dS blocks selects the five-product form
+    // (all of them at once when it holds fa_bwd_fast_workspace_bytes, else for as many K/V heads' groups at a time as
+    // fit, a multiple of eight and not fewer than fa_bwd_min_fast_workspace_bytes allows)
     const unsigned long long fast_bytes = fa_bwd_fast_workspace_bytes(p);
-    a.ds_blocks = (fast_bytes != 0 && p->workspace_bytes >= fast_bytes)
-        ? reinterpret_cast<uint16_t *>(static_cast<char *>(p->workspace) + ds_blocks_offset(p)) : nullptr;
+    a.ds_blocks = nullptr;
+    a.head0 = 0;
+    a.heads = (int)kv_heads_total(p);
+    a.ds_heads = 0;
+    if (fast_bytes != 0 && p->workspace_bytes >= fa_bwd_min_fast_workspace_bytes(p)) {
+        const unsigned long long off = ds_blocks_offset(p);
+        long long fit = (long long)((p->workspace_bytes - off) / ds_bytes_per_kv_head(p));
+        if (fit < kv_heads_total(p)) fit = fit / 8 * 8;
+        a.ds_heads = (int)(fit < kv_heads_total(p) ? fit : kv_heads_total(p));
+        a.ds_blocks = reinterpret_cast<uint16_t *>(static_cast<char *>(p->workspace) + off);
+    }
     a.dQ = static_cast<uint16_t *>(p->dQ);
     a.dK = static_cast<uint16_t *>(p->dK);
     a.dV = static_cast<uint16_t *>(p->dV);

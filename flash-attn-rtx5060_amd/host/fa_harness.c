@@ -223,8 +223,13 @@ int main(int argc, char **argv)
         b.dtype = p.dtype; b.is_causal = c.causal;
         b.alibi_slopes_ptr = p.alibi_slopes_ptr;
         b.dropout_prob = p.dropout_prob; b.seed = p.seed;
-        b.workspace_bytes = fa_bwd_workspace_bytes(&b);
-        if (check(fa_dev_malloc(&ws, (size_t)b.workspace_bytes), "alloc workspace")) return 1;
+        /* the smallest workspace that selects the five-product form (the dS blocks of a chunk of heads), where the
+           problem has that form and the device the memory; else the small one (seven products) */
+        b.workspace_bytes = fa_bwd_min_fast_workspace_bytes(&b);
+        if (b.workspace_bytes == 0 || fa_dev_malloc(&ws, (size_t)b.workspace_bytes) != FA_OK) {
+            b.workspace_bytes = fa_bwd_workspace_bytes(&b);
+            if (check(fa_dev_malloc(&ws, (size_t)b.workspace_bytes), "alloc workspace")) return 1;
+        }
         b.workspace = ws;
         for (int i = 0; i < c.warmup; ++i)
             if (check(fa_bwd(&b, NULL), "backward warm-up launch")) return 1;
@@ -246,8 +251,10 @@ int main(int argc, char **argv)
         const double bmed = ms[c.iters / 2], bbest = ms[0];
         const double bflops = fa_bwd_algorithmic_flops(c.B, c.N, c.S, c.d, c.causal, c.wl, c.wr);
         printf("{\"config\": \"%s backward\", \"iters\": %d, \"ms_median\": %.6f, \"ms_min\": %.6f, \"algorithmic_flops\": %.6e, "
-               "\"tflops_median\": %.3f, \"tflops_best\": %.3f, \"frac_of_peak_median\": %.4f, \"nonfinite_gradients\": %zu}\n",
-               c.name, c.iters, bmed, bbest, bflops, bflops / bmed / 1e9, bflops / bbest / 1e9, bflops / bmed / 1e9 / PEAK_TFLOPS, bad_g);
+               "\"tflops_median\": %.3f, \"tflops_best\": %.3f, \"frac_of_peak_median\": %.4f, \"nonfinite_gradients\": %zu, "
+               "\"workspace_bytes\": %llu}\n",
+               c.name, c.iters, bmed, bbest, bflops, bflops / bmed / 1e9, bflops / bbest / 1e9, bflops / bmed / 1e9 / PEAK_TFLOPS, bad_g,
+               b.workspace_bytes);
         if (bad_g) rc |= 4;
         for (int t = 0; t < 4; ++t) fa_dev_free(dg[t]);
         fa_dev_free(ws);

@@ -63,6 +63,12 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p);
  * workspace plus B*N*S*S storage-type elements (B2 N32 S8192: 8.6 GB).  With it, the key-owning kernel writes every
  * dS block it forms and dQ is one product over those blocks, instead of a second recomputation of S and dP. */
 unsigned long long fa_bwd_fast_workspace_bytes(const fa_bwd_params *p);
+/* The five-product form also runs with less: the dS blocks of as many K/V heads (with their groups of query heads)
+ * at a time as the workspace holds, a multiple of eight, the two kernels launched once per such chunk; same bits as
+ * with the full size.  This is the smallest workspace that selects it (0 when fa_bwd_fast_workspace_bytes is 0):
+ * the small workspace plus the blocks of enough heads for two rounds of key blocks over the chip (B2 N32 S8192:
+ * 16 heads, 2.1 GB).  Anything below it selects the seven-product form. */
+unsigned long long fa_bwd_min_fast_workspace_bytes(const fa_bwd_params *p);
 /* Enqueues the backward pass on `stream` and returns without synchronising: two kernels (dQ and the row sums of
  * dO*O, then dK and dV: seven matrix products), or, with the large workspace, three (the row sums; dK, dV and the
  * dS blocks; dQ from the blocks: five products).  No atomics either way: every output element has one writer and

@@ -128,6 +128,41 @@ def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
 
 
+@pytest.mark.parametrize("B,H,Hk,S,D,dtype,causal,bshd", [(2, 16, 16, 8192, 64, 0, True, False), (6, 16, 8, 4096, 128, 1, True, True),
+                                                          (3, 24, 24, 2048, 128, 0, False, False)])
+def test_five_product_form_in_chunks_of_heads(fa, B, H, Hk, S, D, dtype, causal, bshd):
+    """A workspace that holds the dS blocks of some of the heads only: the key-owning and the query-owning kernel run
+    once per chunk of heads.  Same bits as with the full workspace (every head's arithmetic is the same), with the
+    smallest workspace the form accepts and with one in between whose last chunk is a partial one; one byte less than
+    the smallest selects the seven-product form."""
+    import ctypes
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(77)
+    dt = torch.bfloat16 if dtype else torch.float16
+    q, do = (torch.randn((B, H, S, D), device="cuda", generator=g).to(dt) for _ in range(2))
+    k, v = (torch.randn((B, Hk, S, D), device="cuda", generator=g).to(dt) for _ in range(2))
+    if bshd:
+        q, k, v, do = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v, do))
+    o, lse = fa.flash_attention_forward(q, k, v, causal=causal, exact_first_rows=True)
+    full = fa.flash_attention_backward(q, k, v, o, lse, do, causal=causal, five_products=True, poison_workspace=True)
+    strides = {n: tuple(t.stride()[:3]) for n, t in (("q", q), ("k", k), ("v", v), ("o", o), ("do", do), ("dq", q), ("dk", k), ("dv", v))}
+    p = fa.make_bwd_params(B, H, S, D, causal=causal, dtype=dtype, n_kv_heads=Hk, strides=strides)
+    L = fa.lib()
+    small, least, most = (int(f(ctypes.byref(p))) for f in (L.fa_bwd_workspace_bytes, L.fa_bwd_min_fast_workspace_bytes, L.fa_bwd_fast_workspace_bytes))
+    assert small < least < most
+    for limit in (least, (least + most) // 2):
+        assert limit < most
+        got = fa.flash_attention_backward(q, k, v, o, lse, do, causal=causal, five_products="auto", poison_workspace=True, workspace_limit=limit)
+        torch.cuda.synchronize()
+        for name, x, y in zip(("dQ", "dK", "dV"), full, got):
+            assert torch.equal(x.contiguous().view(torch.int16), y.contiguous().view(torch.int16)), (name, limit)
+    seven = fa.flash_attention_backward(q, k, v, o, lse, do, causal=causal, five_products=False)
+    below = fa.flash_attention_backward(q, k, v, o, lse, do, causal=causal, five_products="auto", workspace_limit=least - 1)
+    torch.cuda.synchronize()
+    for name, x, y in zip(("dQ", "dK", "dV"), seven, below):
+        assert torch.equal(x.contiguous().view(torch.int16), y.contiguous().view(torch.int16)), name
+
+
 FIVE_STRIDED = [
     # B, H, Hk, S, D, dtype, causal, wl, wr, bshd: regular lengths through the strided kernels
     (2, 4, 2, 512, 128, 0, True, -1, -1, True),
