@@ -197,7 +197,9 @@ __device__ __forceinline__ DropWords dropout_words(uint32_t seed_lo, uint32_t se
         // of which runs at a quarter of the vector ALU's rate)
         const uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c0, p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
         const uint32_t h0 = (uint32_t)(p0 >> 32), l0 = (uint32_t)p0, h1 = (uint32_t)(p1 >> 32), l1 = (uint32_t)p1;
-        c0 = h1 ^ c1 ^ k0; c1 = l1; c2 = h0 ^ c3 ^ k1; c3 = l0;
+        // (the two three-way exclusive ors as one v_bitop3_b32 each, truth table 0x96; left to the compiler they
+        // are two v_xor_b32 each)
+        c0 = __builtin_amdgcn_bitop3_b32(h1, c1, k0, 0x96); c1 = l1; c2 = __builtin_amdgcn_bitop3_b32(h0, c3, k1, 0x96); c3 = l0;
         k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
     }
     return DropWords{{c0, c1, c2, c3}};
@@ -801,7 +803,9 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     };
     auto dropped = [&](float e, int kb, int r) __attribute__((always_inline)) {
         if (!DROPOUT) return e;
-        return dropout_keep_byte(dw[kb], r, a.drop_threshold) ? e * a.drop_scale : 0.0f;
+        // (a kept probability's factor 1 / (1 - p) is the same for all of them: it multiplies the row once, in the
+        // epilogue, instead of 32 elements per lane and tile here)
+        return dropout_keep_byte(dw[kb], r, a.drop_threshold) ? e : 0.0f;
     };
     auto softmax_plain = [&](int tile) __attribute__((always_inline)) {
         if (DROPOUT) draw_dropout(tile);
@@ -1131,7 +1135,7 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
             const float l_half = l_a + l_b;
             const float l_tot = l_half + swap_halves(l_half);
             const bool empty = GENERAL && !(l_tot > 0.0f);         // this row saw no key (here)
-            const float inv = empty ? 0.0f : 1.0f / l_tot;
+            const float inv = empty ? 0.0f : (DROPOUT ? a.drop_scale : 1.0f) / l_tot;
             const float lse_row = empty ? -INFINITY
                                         : m_run * a.scale + __builtin_logf(l_tot);
             if (GENERAL && o_part != nullptr) {
