@@ -47,6 +47,9 @@ hipError_t fa_configure_forward_dropout();
 hipError_t fa_configure_forward_dropout_regular();
 hipError_t fa_configure_backward();
 hipError_t fa_configure_backward_dropout();
+hipError_t fa_launch_backward_dropout_regular(const FaBwdArgs &a, int bf16, int D, int masked, int strided, int compute_units,
+                                              hipStream_t stream, bool configure_only = false);
+hipError_t fa_configure_backward_dropout_regular();
 hipError_t fa_configure_backward_strided();
 
 namespace {
@@ -493,7 +496,7 @@ int fa_init(void)
     // a HIP call on this device that is not a stream operation (which is what a stream capture needs)
     hipError_t (*const configure[])() = {fa_configure_forward_contiguous, fa_configure_forward_strided, fa_configure_forward_general,
                                          fa_configure_forward_dropout, fa_configure_forward_dropout_regular, fa_configure_backward, fa_configure_backward_dropout,
-                                         fa_configure_backward_strided};
+                                         fa_configure_backward_strided, fa_configure_backward_dropout_regular};
     for (auto fn : configure) {
         e = fn();
         if (e != hipSuccess) return device_fail(e, "kernel set-up");
@@ -664,11 +667,11 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
 
 namespace {
 // what the contiguous and the strided kernels run: S a multiple of 128 and as many keys, in any storage order and
-// with any grouping of K/V heads; no ALiBi, no dropout
+// with any grouping of K/V heads, with or without dropout; no ALiBi
 bool five_product_shape(const fa_bwd_params *p)
 {
     if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S)) return false;
-    return p->alibi_slopes_ptr == nullptr && !(fa_dropout_threshold(p->dropout_prob) != 0);
+    return p->alibi_slopes_ptr == nullptr;
 }
 unsigned long long ds_blocks_offset(const fa_bwd_params *p)
 {
@@ -811,7 +814,10 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.seed_lo = (unsigned)(p->seed & 0xffffffffull);
     a.seed_hi = (unsigned)(p->seed >> 32);
     const int masked = (general || a.L < far || a.R < far) ? 1 : 0;
-    hipError_t e = a.drop_threshold != 0
+    hipError_t e = (a.drop_threshold != 0 && !general)
+        ? fa_launch_backward_dropout_regular(a, p->dtype == FA_DTYPE_BF16, p->d, masked, strided ? 1 : 0, ds->compute_units,
+                                             static_cast<hipStream_t>(stream))
+        : a.drop_threshold != 0
         ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, ds->compute_units,
                                      static_cast<hipStream_t>(stream))
         : (strided && !general)

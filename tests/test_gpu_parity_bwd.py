@@ -115,16 +115,16 @@ def test_five_product_form_against_the_fp64_oracle(fa, oracle, shape, dtype, cau
 
 def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
     """Lengths a multiple of 128 with as many keys, in any storage order and with any grouping of K/V heads (the dS
-    blocks are per QUERY head); not with other lengths, ALiBi or dropout."""
+    blocks are per QUERY head), with or without dropout; not with other lengths or ALiBi."""
     import ctypes
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128)
     small = L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok)))
     large = ((small + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
     assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == large
-    for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)})):
+    for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)}), dict(dropout_prob=0.1)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **same}))) == large, same
-    for other in (dict(S=1000), dict(S_kv=2048), dict(dropout_prob=0.1), dict(alibi_ptr=256)):
+    for other in (dict(S=1000), dict(S_kv=2048), dict(alibi_ptr=256)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
 
 
@@ -383,13 +383,20 @@ DROPOUT = [
     (1, 2, 2, 200, 456, 128, 1, True, -1, -1, False, False, 0.5, 7),                     # more keys than queries, bf16
     (1, 2, 1, 190, 190, 64, 0, False, 50, 30, True, False, 0.2, 8),                      # ALiBi, window, one K/V head
     (1, 3, 3, 640, 640, 128, 0, True, 100, -1, True, False, 0.9, 9),                     # almost everything dropped
+    # regular lengths without ALiBi: kernels of their own, with a five-product form
+    (2, 4, 2, 512, 512, 128, 1, True, -1, -1, False, True, 0.3, 10),                      # grouped heads, [B,S,H,D]
+    (1, 2, 2, 640, 640, 64, 0, False, 64, 40, False, False, 0.1, 11),
+    (1, 3, 1, 384, 384, 128, 0, True, 200, -1, False, True, 0.6, 12),
 ]
 
 
+@pytest.mark.parametrize("five", [False, True])
 @pytest.mark.parametrize("B,H,Hk,S,Skv,D,dtype,causal,wl,wr,alibi,bshd,p,seed", DROPOUT)
-def test_dropout_gradients_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd, p, seed):
+def test_dropout_gradients_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv, D, dtype, causal, wl, wr, alibi, bshd, p, seed, five):
     """The backward pass replays the forward's keep decisions from (seed, head, query position, key); the oracle
-    does the same on the CPU.  Kept probabilities are multiplied by 1/(1-p), and so is every rounding error."""
+    does the same on the CPU.  Kept probabilities are multiplied by 1/(1-p), and so is every rounding error.
+    Both forms: with five products (regular lengths without ALiBi; the others run seven either way) only the
+    key-owning kernel replays the decisions, and the workspace is filled with NaN first."""
     import torch
     thr = fa.lib().fa_dropout_threshold(p)
     q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=800 + S)
@@ -403,8 +410,8 @@ def test_dropout_gradients_against_the_fp64_oracle(fa, oracle, B, H, Hk, S, Skv,
     ts = None if slopes is None else torch.from_numpy(slopes).cuda()
     kw = dict(causal=causal, window_left=wl, window_right=wr, alibi_slopes=ts, dropout_prob=p, seed=seed)
     o, lse = fa.flash_attention_forward(tq, tk, tv, **kw)
-    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
-    dq2, dk2, dv2 = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, **kw)
+    dq, dk, dv = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products=five, poison_workspace=True, **kw)
+    dq2, dk2, dv2 = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products=five, poison_workspace=True, **kw)
     torch.cuda.synchronize()
     grow = 256.0 / (256 - thr)
     rel, mx = (1e-3, 2e-3) if dtype == 0 else (8e-3, 1.6e-2)
