@@ -172,8 +172,8 @@ def backward_bench(args):
         err[name] = {"rel_l2": float(d.norm() / want.norm()), "max_abs": float(d.abs().max()), "max_ref": float(want.abs().max())}
     tf = flops / (wall_ms * 1e-3) / 1e12
     plain = args.dropout == 0 and args.layout == "bhsd" and not args.kv_heads and not args.alibi      # the reference's layout
-    # (the five-product form exists for regular lengths in any storage order and head grouping, with or without dropout, not with ALiBi)
-    form = "five" if (args.bwd_form == "five" and not args.alibi and S % 128 == 0) else "seven"
+    # (the five-product form exists for regular lengths in any storage order and head grouping, with dropout or with ALiBi, not with both)
+    form = "five" if (args.bwd_form == "five" and not (args.alibi and args.dropout > 0) and S % 128 == 0) else "seven"
     print(json.dumps({
         "metric": "attn backward TFLOPS (dQ, dK, dV), 1 GPU", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,

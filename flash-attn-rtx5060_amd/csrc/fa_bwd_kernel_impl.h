@@ -189,7 +189,6 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
     static_assert(LAYOUT >= 0 && LAYOUT <= 2, "0 the reference's layout, 1 strided, 2 general");
     static_assert(!GENERAL || MASKED, "the general instantiations always carry the mask code (ragged tiles need it)");
-    static_assert(!ALIBI || GENERAL, "ALiBi is instantiated for the general layout only");
 
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
@@ -390,7 +389,7 @@ template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, b
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
     constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
-    static_assert(!WRITE_DS || (LAYOUT <= 1 && !ALIBI), "dS blocks are written for regular lengths without ALiBi only");
+    static_assert(!WRITE_DS || LAYOUT <= 1, "dS blocks are written for regular lengths only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
@@ -512,7 +511,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // value the compiler spills to scratch memory inside the tile loop comes back behind a wait for ALL loads and
     // stores in flight.  The last PARKED of the K^T and V^T fragments, which every half tile uses once, are kept in
     // LDS instead (32 bytes per lane and fragment pair, written once per work item) and read like any A operand.
-    constexpr int PARKED = WRITE_DS && D == 128 ? (DROPOUT ? FA_PARK_DROP : 1) : 0;
+    constexpr int PARKED = WRITE_DS && D == 128 ? (DROPOUT ? FA_PARK_DROP : ALIBI ? 2 : 1) : 0;
     constexpr uint32_t kParkPlane = 16u * kBwdWaves * 64u;
     const uint32_t park_lds = lds0 + NSTG * STAGEB + (DROPOUT ? kBwdWaves * 128 : 0);       // (behind the dropout words)
     auto parked = [&](int which, int s) __attribute__((always_inline)) {
@@ -922,11 +921,11 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
     a.head0 = 0;
     a.heads = all_heads;
     const int smem_dq = kBwdStages * 2 * TILEB, smem_dkdv = kBwdStages * (2 * TILEB + 512) + (DROPOUT ? kBwdWaves * 128 : 0);
-    const int smem_dkdv_ds = smem_dkdv + (D == 128 ? (DROPOUT ? FA_PARK_DROP : 1) * 32 * kBwdWaves * 64 : 0);      // + the parked fragments
+    const int smem_dkdv_ds = smem_dkdv + (D == 128 ? (DROPOUT ? FA_PARK_DROP : ALIBI ? 2 : 1) * 32 * kBwdWaves * 64 : 0);      // + the parked fragments
     auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
     auto kkv = fa_bwd_dkdv<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
-    // the five-product form: regular lengths (the reference's layout or a strided one), no ALiBi
-    constexpr bool FIVE = LAYOUT <= 1 && !ALIBI;
+    // the five-product form: regular lengths (the reference's layout or a strided one)
+    constexpr bool FIVE = LAYOUT <= 1;
     constexpr int FL = FIVE ? LAYOUT : 0;
     const int smem_dq_ds = kBwdStages * (TILEB + kBwdWaves * 2 * kDsBlockBytes);
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
@@ -938,7 +937,7 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kkv), hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv);
         if (e != hipSuccess) return e;
         if constexpr (FIVE) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, FL, false, DROPOUT, true>),
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, FL, ALIBI, DROPOUT, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv_ds);
             if (e != hipSuccess) return e;
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>),
@@ -981,7 +980,7 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
                 a.heads = all_heads - h0 < chunk ? all_heads - h0 : chunk;
                 const unsigned launch_k = grid_for((long long)a.heads * ((a.Sk + 255) / 256));
                 const unsigned launch_q = grid_for((long long)a.heads * group * ((a.S + 255) / 256));
-                hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, false, DROPOUT, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
+                hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, ALIBI, DROPOUT, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
                 hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
             }
             return hipGetLastError();

@@ -50,6 +50,9 @@ hipError_t fa_configure_backward_dropout();
 hipError_t fa_launch_backward_dropout_regular(const FaBwdArgs &a, int bf16, int D, int masked, int strided, int compute_units,
                                               hipStream_t stream, bool configure_only = false);
 hipError_t fa_configure_backward_dropout_regular();
+hipError_t fa_launch_backward_alibi_regular(const FaBwdArgs &a, int bf16, int D, int masked, int strided, int compute_units,
+                                            hipStream_t stream, bool configure_only = false);
+hipError_t fa_configure_backward_alibi_regular();
 hipError_t fa_configure_backward_strided();
 
 namespace {
@@ -496,7 +499,7 @@ int fa_init(void)
     // a HIP call on this device that is not a stream operation (which is what a stream capture needs)
     hipError_t (*const configure[])() = {fa_configure_forward_contiguous, fa_configure_forward_strided, fa_configure_forward_general,
                                          fa_configure_forward_dropout, fa_configure_forward_dropout_regular, fa_configure_backward, fa_configure_backward_dropout,
-                                         fa_configure_backward_strided, fa_configure_backward_dropout_regular};
+                                         fa_configure_backward_strided, fa_configure_backward_dropout_regular, fa_configure_backward_alibi_regular};
     for (auto fn : configure) {
         e = fn();
         if (e != hipSuccess) return device_fail(e, "kernel set-up");
@@ -667,11 +670,11 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
 
 namespace {
 // what the contiguous and the strided kernels run: S a multiple of 128 and as many keys, in any storage order and
-// with any grouping of K/V heads, with or without dropout; no ALiBi
+// with any grouping of K/V heads, with dropout or with ALiBi (both at once run the general kernels)
 bool five_product_shape(const fa_bwd_params *p)
 {
     if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S)) return false;
-    return p->alibi_slopes_ptr == nullptr;
+    return !(p->alibi_slopes_ptr != nullptr && fa_dropout_threshold(p->dropout_prob) != 0);
 }
 unsigned long long ds_blocks_offset(const fa_bwd_params *p)
 {
@@ -785,7 +788,8 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     a.S = p->S;
     a.Sk = p->S_kv > 0 ? p->S_kv : p->S;
     // general: any lengths, ALiBi, dropout; strided: the reference's lengths with other strides or grouped K/V heads
-    const bool general = a.S % 128 != 0 || a.Sk != a.S || a.alibi != nullptr;
+    // (drop_threshold is set further down: the same function of the probability)
+    const bool general = a.S % 128 != 0 || a.Sk != a.S || (a.alibi != nullptr && fa_dropout_threshold(p->dropout_prob) != 0);
     bool strided = a.Hk != a.H;
     {
         const long long *strides[8] = {p->q_strides, p->k_strides, p->v_strides, p->o_strides, p->do_strides,
@@ -817,6 +821,9 @@ int fa_bwd(const fa_bwd_params *p, void *stream)
     hipError_t e = (a.drop_threshold != 0 && !general)
         ? fa_launch_backward_dropout_regular(a, p->dtype == FA_DTYPE_BF16, p->d, masked, strided ? 1 : 0, ds->compute_units,
                                              static_cast<hipStream_t>(stream))
+        : (a.alibi != nullptr && !general)
+        ? fa_launch_backward_alibi_regular(a, p->dtype == FA_DTYPE_BF16, p->d, masked, strided ? 1 : 0, ds->compute_units,
+                                           static_cast<hipStream_t>(stream))
         : a.drop_threshold != 0
         ? fa_launch_backward_dropout(a, p->dtype == FA_DTYPE_BF16, p->d, a.alibi != nullptr ? 1 : 0, ds->compute_units,
                                      static_cast<hipStream_t>(stream))

@@ -115,16 +115,17 @@ def test_five_product_form_against_the_fp64_oracle(fa, oracle, shape, dtype, cau
 
 def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
     """Lengths a multiple of 128 with as many keys, in any storage order and with any grouping of K/V heads (the dS
-    blocks are per QUERY head), with or without dropout; not with other lengths or ALiBi."""
+    blocks are per QUERY head), with dropout or with ALiBi; not with other lengths, nor with both options at once."""
     import ctypes
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128)
     small = L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok)))
     large = ((small + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
     assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ok))) == large
-    for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)}), dict(dropout_prob=0.1)):
+    for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)}), dict(dropout_prob=0.1),
+                 dict(alibi_ptr=256)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **same}))) == large, same
-    for other in (dict(S=1000), dict(S_kv=2048), dict(alibi_ptr=256)):
+    for other in (dict(S=1000), dict(S_kv=2048), dict(alibi_ptr=256, dropout_prob=0.1)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
 
 
@@ -176,23 +177,45 @@ FIVE_STRIDED = [
 
 @pytest.mark.parametrize("B,H,Hk,S,D,dtype,causal,wl,wr,bshd", FIVE_STRIDED)
 def test_five_product_form_in_strided_layouts_and_with_grouped_heads(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd):
-    """The five-product form through the strided kernels ([B,S,H,D] storage, K/V heads shared by groups of query
-    heads: the key-owning workgroup writes the dS blocks of every query head of its group), against the fp64 oracle
-    and with a NaN-filled workspace, twice with the same bits; the seven-product form of the same call meets the same bars."""
+    """[B,S,H,D] storage and K/V heads shared by groups of query heads: the key-owning workgroup writes the dS blocks
+    of every query head of its group."""
+    five_product_case(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd, False)
+
+
+ALIBI_REGULAR = [
+    # B, H, Hk, S, D, dtype, causal, wl, wr, bshd: regular lengths with ALiBi slopes of both signs
+    (1, 4, 4, 384, 128, 0, True, -1, -1, False),
+    (2, 4, 2, 512, 128, 1, True, 200, -1, True),
+    (1, 2, 2, 256, 64, 0, False, -1, -1, False),
+    (1, 6, 2, 640, 64, 0, False, 50, 30, True),
+    (1, 2, 1, 768, 128, 0, False, -1, -1, True),
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,D,dtype,causal,wl,wr,bshd", ALIBI_REGULAR)
+def test_alibi_on_regular_lengths_in_both_forms(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd):
+    """ALiBi on regular lengths runs kernels of its own (not the general ones), in both storage orders, with the
+    five-product form: the bias enters the score the key-owning kernel recomputes, dS carries it from there."""
+    five_product_case(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd, True)
+
+
+def five_product_case(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd, alibi):
+    """The five-product form against the fp64 oracle, with a NaN-filled workspace, twice with the same bits; the
+    seven-product form of the same call meets the same bars."""
     import torch
     q, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=720 + S)
     do, _, _ = make_inputs(fa, (B, H, S, D), dtype, seed=721 + S)
     _, k, v = make_inputs(fa, (B, Hk, S, D), dtype, seed=722 + S)
-    dq_ref, dk_ref, dv_ref = oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, None)
+    slopes = (np.power(2.0, -8.0 / H * (np.arange(H) + 1)) * np.where(np.arange(H) % 2, -0.5, 1.0)).astype(np.float32) if alibi else None
+    dq_ref, dk_ref, dv_ref = oracle_bwd_general(oracle, q, k, v, do, dtype, causal, wl, wr, slopes)
     tq, tk, tv, tdo = (to_torch(x, dtype) for x in (q, k, v, do))
     if bshd:
         tq, tk, tv, tdo = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (tq, tk, tv, tdo))
-    o, lse = fa.flash_attention_forward(tq, tk, tv, causal=causal, window_left=wl, window_right=wr, exact_first_rows=True)
-    five = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=True,
-                                       poison_workspace=True)
-    seven = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=False)
-    again = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, causal=causal, window_left=wl, window_right=wr, five_products=True,
-                                        poison_workspace=True)
+    kw = dict(causal=causal, window_left=wl, window_right=wr, alibi_slopes=None if slopes is None else torch.from_numpy(slopes).cuda())
+    o, lse = fa.flash_attention_forward(tq, tk, tv, exact_first_rows=True, **kw)
+    five = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products=True, poison_workspace=True, **kw)
+    seven = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products=False, **kw)
+    again = fa.flash_attention_backward(tq, tk, tv, o, lse, tdo, five_products=True, poison_workspace=True, **kw)
     torch.cuda.synchronize()
     for name, got, want, other, rerun, like in zip(("dQ", "dK", "dV"), five, (dq_ref, dk_ref, dv_ref), seven, again, (tq, tk, tv)):
         assert got.stride() == like.stride()
