@@ -15,8 +15,10 @@
 // Template flags: LAYOUT 0 = contiguous [B,H,S,D] with S a multiple of 128 and as many keys; 1 (strided) = the
 // same lengths with row, head and batch strides from the arguments and grouped K/V heads; 2 (general) = that
 // plus any lengths (query i at key position i + Sk - S, ragged last tiles).  Each keeps its instruction stream
-// free of what it does not need.  ALIBI (general only) subtracts slope[h] * |position - key| from the scaled
-// score.  DROPOUT (general only) replays the forward pass's keep decisions from (seed, head, query position, key).
+// free of what it does not need.  ALIBI subtracts slope[h] * |position - key| from the scaled score.  DROPOUT
+// replays the forward pass's keep decisions from (seed, head, query position, key).  (Either one is instantiated
+// for all three layouts, both together for the general one only.)
+// Layouts 0 and 1 also have a five-product form (fa_bwd_prepare, fa_bwd_dkdv<WRITE_DS>, fa_bwd_dq_from_ds below).
 // Both walkers use the building blocks of the forward kernel: 32x32x16 MFMA with the thing a wave owns on the
 // lane (query in fa_bwd_dq, key in fa_bwd_dkdv), so that the owner's operands are B operands loaded once into
 // registers, the walked tiles are A operands streamed through LDS by direct global->LDS loads, and an
