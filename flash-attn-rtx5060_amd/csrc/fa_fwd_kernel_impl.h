@@ -1077,13 +1077,16 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     const bool faithful = first_rows_on && q0 == 0;         // this item's own rows 0..31 are not stored by the epilogue
     const int f_rows = !faithful ? 0 : !GENERAL ? kFaithfulRows : (kFaithfulRows - pos_off < S ? kFaithfulRows - pos_off : S);
     // Which of those rows THIS item recomputes.  General layouts: the item with the head's first block, all of
-    // them.  Contiguous layout: the 32 rows are dealt in 2 or 4 parts to the head's first query blocks, one
+    // them.  Contiguous layout: the 32 rows are dealt in 2, 4 or 8 parts to the head's first query blocks, one
     // part each -- under a static schedule the workgroups that run the path are the critical path of a short
-    // problem (c2: 64 of 256 workgroups carried 7.7 us each), and every pair of items of the snake then gets one.
+    // problem (c2: 64 of 256 workgroups carried 7.7 us each), and every pair of items of the snake then gets one
+    // (eight parts for heads of sixteen blocks or more under the static schedules, where the snake pairs block
+    // 15 with 0, 14 with 1, ... 8 with 7: c2 592.7 against 584.4 TFLOP/s, B4 H32 S2048 D64 654.7 against 641.7; the
+    // work queue balances by itself and keeps four larger parts).
     int fr0 = 0, fr1 = 0;
     if (GENERAL) fr1 = f_rows;
     else if (first_rows_on) {
-        const int parts = a.n_qblocks >= 4 ? 4 : a.n_qblocks >= 2 ? 2 : 1;
+        const int parts = (a.n_qblocks >= 16 && a.queue == nullptr) ? 8 : a.n_qblocks >= 4 ? 4 : a.n_qblocks >= 2 ? 2 : 1;
         if (qblock < parts) { fr0 = qblock * (kFaithfulRows / parts); fr1 = fr0 + kFaithfulRows / parts; }
     }
     // ---- the next work item, and the first requests for it
