@@ -1079,14 +1079,20 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     // Which of those rows THIS item recomputes.  General layouts: the item with the head's first block, all of
     // them.  Contiguous layout: the 32 rows are dealt in 2, 4 or 8 parts to the head's first query blocks, one
     // part each -- under a static schedule the workgroups that run the path are the critical path of a short
-    // problem (c2: 64 of 256 workgroups carried 7.7 us each), and every pair of items of the snake then gets one
-    // (eight parts for heads of sixteen blocks or more under the static schedules, where the snake pairs block
-    // 15 with 0, 14 with 1, ... 8 with 7: c2 592.7 against 584.4 TFLOP/s, B4 H32 S2048 D64 654.7 against 641.7; the
-    // work queue balances by itself and keeps four larger parts).
+    // problem (c2: 64 of 256 workgroups carried 7.7 us each), and every pair of items of the snake then gets one:
+    // as many parts as half the head's blocks (at most eight), since the snake pairs block n - 1 with 0, n - 2 with
+    // 1, ...  (Eight parts instead of four at sixteen blocks: c2 592.7 against 584.4 TFLOP/s, B4 H32 S2048 D64 654.7
+    // against 641.7; two parts instead of four at four blocks, where four gave every pair two of them: causal B16 H16
+    // S512 D128 380.1 against 359.3, D64 276.8 against 266.3.)  One workgroup per item and the work queue, which
+    // balances by itself, keep four parts.
     int fr0 = 0, fr1 = 0;
     if (GENERAL) fr1 = f_rows;
     else if (first_rows_on) {
-        const int parts = (a.n_qblocks >= 16 && a.queue == nullptr) ? 8 : a.n_qblocks >= 4 ? 4 : a.n_qblocks >= 2 ? 2 : 1;
+        // (a resident grid without a queue walks the list as a snake: a workgroup's items come in pairs of block k
+        // and block n - 1 - k, and parts on the lower half of the blocks give every pair exactly one)
+        const bool snake = a.queue == nullptr && (long long)gridDim.x < a.n_items;
+        const int parts = snake ? (a.n_qblocks >= 16 ? 8 : a.n_qblocks >= 8 ? 4 : a.n_qblocks >= 4 ? 2 : 1)
+                                : (a.n_qblocks >= 4 ? 4 : a.n_qblocks >= 2 ? 2 : 1);
         if (qblock < parts) { fr0 = qblock * (kFaithfulRows / parts); fr1 = fr0 + kFaithfulRows / parts; }
     }
     // ---- the next work item, and the first requests for it
