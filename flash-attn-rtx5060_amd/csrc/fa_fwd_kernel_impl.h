@@ -1086,7 +1086,13 @@ __global__ void __launch_bounds__(NW * 64, 2) fa_fwd_pipelined(const FaKernelArg
     // S512 D128 380.1 against 359.3, D64 276.8 against 266.3.)  One workgroup per item and the work queue, which
     // balances by itself, keep four parts.
     int fr0 = 0, fr1 = 0;
-    if (GENERAL) fr1 = f_rows;
+    // (general layouts deal the rows the same way when the problem is the plain one at another length: queries
+    // that start at key position 0, no key splits; otherwise the item with the head's first block keeps them all)
+    // (causal B8 H32 S1000 D64 445 against 382 TFLOP/s, B16 H16 S500 D128 341 against 296, B4 H16 S2047 D64 573 against
+    // 521.  The general 4-wave kernels keep two LDS stages per tensor: with three for K their 128-wide instantiations
+    // spill 24-40 bytes and measure 3-5 % slower.)
+    const bool dealt = !GENERAL || (n_splits == 1 && pos_off == 0 && a.n_qblocks >= 2);
+    if (!dealt) fr1 = f_rows;
     else if (first_rows_on) {
         // (a resident grid without a queue walks the list as a snake: a workgroup's items come in pairs of block k
         // and block n - 1 - k, and parts on the lower half of the blocks give every pair exactly one)

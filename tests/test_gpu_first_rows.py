@@ -31,7 +31,12 @@ def ulp(x, dtype):
                                                  # rows, under every schedule (several passes over the resident grid included)
                                                  ((1, 4, 128, 64), -1, 5, 0), ((1, 4, 512, 128), -1, 6, 2), ((4, 64, 2048, 64), -1, 28, 0),
                                                  ((4, 64, 2048, 64), 40, 28, 3), ((8, 80, 768, 128), -1, 9, 2), ((8, 80, 512, 64), -1, 10, 3),
-                                                 ((8, 80, 256, 64), -1, 11, 1)])
+                                                 ((8, 80, 256, 64), -1, 11, 1),
+                                                 # other lengths (the general kernels deal the rows the same way): two, four
+                                                 # and eight parts, one block alone, every schedule
+                                                 ((2, 8, 200, 128), -1, 12, 0), ((4, 64, 500, 64), -1, 13, 2), ((4, 64, 1000, 128), -1, 14, 0),
+                                                 ((4, 64, 2047, 64), 100, 15, 2), ((2, 16, 1100, 128), -1, 16, 3), ((8, 80, 300, 64), -1, 17, 1),
+                                                 ((1, 4, 100, 128), -1, 18, 0)])
 def test_first_rows_are_the_verifiers_bits(fa, oracle, dtype, shape, wl, seed, sched):
     B, H, S, D = shape
     q, k, v = make_inputs(fa, shape, dtype, seed)
