@@ -333,8 +333,8 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     ``five_products``: True asks for the workspace that selects the five-product form (fa_bwd_fast_workspace_bytes:
     B*N*S*S elements more), False for the small one; "auto" takes, when the problem qualifies, the dS blocks of about
     2 GiB worth of heads (the form then runs over the heads in chunks, which measures no slower), at least
-    fa_bwd_min_fast_workspace_bytes and at most a quarter of the device's free memory, or ``workspace_limit`` bytes
-    when that is given; when even the least does not fit, the small one.  ``poison_workspace`` (for tests) fills the workspace with
+    fa_bwd_min_fast_workspace_bytes and at most ``workspace_limit`` bytes when that is given; when the device has no
+    room for it, the least, and when not for that either, the small one.  ``poison_workspace`` (for tests) fills the workspace with
     NaN bit patterns first: the kernels must not read anything in it that they have not written.
     Shapes and strides as in flash_attention_forward (q, o, do [B, N, S, d]; k, v [B, Nk, S_kv, d]; lse
     [B, N, S] float32 contiguous); dq, dk, dv come back with the strides of q, k, v."""
@@ -372,28 +372,38 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
                         n_kv_heads=0 if Nk == N else Nk, S_kv=0 if S_kv == S else S_kv,
                         alibi_ptr=0 if alibi_slopes is None else alibi_slopes.data_ptr(), strides=strides,
                         dropout_prob=dropout_prob, seed=seed)
-    need = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
+    small = lib().fa_bwd_workspace_bytes(ctypes.byref(p))
     fast = lib().fa_bwd_fast_workspace_bytes(ctypes.byref(p)) if five_products else 0
+    sizes = [small]                       # tried from the back; the small workspace is what is left when nothing else fits
     if fast and five_products is True and workspace_limit is None:
-        need = fast
+        sizes.append(fast)
     elif fast:
         # "auto": whole chunks of eight K/V heads' dS blocks, about 2 GiB of them (chunks measure no slower than the
         # full size: B2 N32 S8192 D128 3.27 ms with 2.2 or 4.4 GB against 3.34 with 8.6), never fewer heads than the
-        # library accepts and never more bytes than the limit; a size that depends on the problem alone, so that
-        # torch's allocator hands the same block back call after call
+        # library accepts and never more bytes than the limit; sizes that depend on the problem alone, so that
+        # torch's allocator hands the same block back call after call (and no query of the device's free memory:
+        # torch's memory statistics cost a millisecond per call, ten times a short problem's backward pass)
         least = lib().fa_bwd_min_fast_workspace_bytes(ctypes.byref(p))
-        off = (need + 255) // 256 * 256
+        off = (small + 255) // 256 * 256
         kv_total = q.shape[0] * k.shape[1]
         per_head = (fast - off) // kv_total
         heads = max((least - off) // per_head, (2 << 30) // per_head // 8 * 8)
-        limit = workspace_limit if workspace_limit is not None else _ws_budget(q.device)
+        limit = workspace_limit if workspace_limit is not None else fast
         if off + heads * per_head > limit:
             heads = (limit - off) // per_head // 8 * 8 if limit > off else 0
-        if heads >= kv_total and fast <= limit:
-            need = fast
-        elif heads > 0 and off + heads * per_head >= least:
-            need = off + heads * per_head
-    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)     # stream-ordered: freed after the launch
+        want = fast if heads >= kv_total else off + heads * per_head
+        if least <= limit and want > least:
+            sizes.append(least)
+        if heads > 0 and least <= want <= limit:
+            sizes.append(want)
+    workspace = None
+    while workspace is None:              # stream-ordered: freed after the launch
+        need = sizes.pop()
+        try:
+            workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+        except torch.cuda.OutOfMemoryError:
+            if not sizes:
+                raise
     if poison_workspace:
         workspace.fill_(0xff)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), need
@@ -401,14 +411,6 @@ def flash_attention_backward(q, k, v, o, lse, do, softmax_scale=None, causal=Fal
     if st != FA_OK:
         raise FaError(st, lib().fa_last_device_error().decode() if st == FA_ERR_DEVICE else "")
     return dq, dk, dv
-
-
-def _ws_budget(device):
-    """A quarter of the memory a new allocation could get: the device's free memory plus what torch's allocator
-    holds without using it."""
-    import torch
-    free, _ = torch.cuda.mem_get_info(device)
-    return (free + torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)) // 4
 
 
 _autograd_function = None

@@ -188,7 +188,7 @@ __device__ __forceinline__ uint16_t *head_ptr(uint16_t *p, const FaBwdTensor &t,
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a)
 {
-    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
+    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES && D == 128;
     static_assert(LAYOUT >= 0 && LAYOUT <= 2, "0 the reference's layout, 1 strided, 2 general");
     static_assert(!GENERAL || MASKED, "the general instantiations always carry the mask code (ragged tiles need it)");
 
@@ -205,7 +205,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
     // Work items: one workgroup per item, or (grid smaller than the list) a resident grid that walks the
     // longest-first list as a snake, pass 0 forwards, pass 1 backwards, ..., which pairs long items with short ones.
     const long long n_items = (long long)a.B * a.H * n_qblocks;
-    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (strided and general instantiations: exactly one item, no loop)
+    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (128-wide strided and general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();          // (the LDS stages: other waves may still be reading the last tile)
@@ -390,7 +390,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, bool WRITE_DS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
-    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES;
+    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES && D == 128;
     static_assert(!WRITE_DS || LAYOUT <= 1, "dS blocks are written for regular lengths only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
@@ -407,7 +407,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
     // (work items as in fa_bwd_dq; the list here is ascending in the key block, which is longest first under a
     // causal mask: key block 0 is seen by every query)
     const long long n_items = (long long)a.heads * n_kblocks;
-    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (strided and general instantiations: exactly one item, no loop)
+    for (int pass = 0; !ONE_ITEM || pass < 1; ++pass) {       // (128-wide strided and general instantiations: exactly one item, no loop)
     const long long item = (long long)pass * gridDim.x + ((pass & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
     if (item >= n_items) break;
     if (pass > 0) __syncthreads();
@@ -961,10 +961,10 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
     // (the general instantiations always carry the mask code: without a bound on either side, L = R = S + S_kv, their
     // items are alike as well)
     const long long unbounded = (long long)a.S + a.Sk;
-    // (The strided and general instantiations are launched one workgroup per item only: with the item loop around
-    // them their 128-wide kernels spill ten times as much, and a reload inside the tile loop waits for every tile
-    // load in flight: c3's shape stored [B,S,H,D] 4.1 ms against 3.8.)
-    const bool uneven = LAYOUT == 0 && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
+    // (The 128-wide strided and general instantiations are launched one workgroup per item only: with the item loop
+    // around them they spill ten times as much, and a reload inside the tile loop waits for every tile load in
+    // flight: c3's shape stored [B,S,H,D] 4.1 ms against 3.8.  The 64-wide ones have the registers for the loop.)
+    const bool uneven = (LAYOUT == 0 || D == 64) && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
     auto grid_for = [&](long long items) {
         const unsigned g = (unsigned)items;
         return (uneven && g > resident && g < 16u * resident) ? resident : g;
