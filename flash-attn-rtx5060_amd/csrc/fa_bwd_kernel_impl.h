@@ -391,7 +391,7 @@ template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, b
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
     constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES && D == 128;
-    static_assert(!WRITE_DS || LAYOUT <= 1, "dS blocks are written for regular lengths only");
+    static_assert(!WRITE_DS || LAYOUT <= 1 || (!ALIBI && !DROPOUT), "general lengths: dS blocks without ALiBi and dropout only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
@@ -617,7 +617,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs
             const uint64_t ub = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(dst >> 32)) << 32) |
                                 (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)dst);
             const uint32_t voff = 16u * __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-            const u32x4 w0 = {pp[0], pp[1], pp[2], pp[3]}, w1 = {pp[4], pp[5], pp[6], pp[7]};
+            u32x4 w0 = {pp[0], pp[1], pp[2], pp[3]}, w1 = {pp[4], pp[5], pp[6], pp[7]};
+            // (general lengths: a lane whose key lies past the end has worked on a copy of the last key; what the
+            // query-owning kernel multiplies with the padding rows of its last key tile must be zero)
+            if (GENERAL && my_k >= Sk) { w0 = u32x4{0, 0, 0, 0}; w1 = u32x4{0, 0, 0, 0}; }
             asm volatile("global_store_dwordx4 %0, %1, %3 nt\n\tglobal_store_dwordx4 %0, %2, %3 offset:1024 nt\n\ts_nop 1"
                          :: "v"(voff), "v"(w0), "v"(w1), "s"(ub) : "memory");
         }
@@ -777,9 +780,10 @@ __global__ void __launch_bounds__(256) fa_bwd_prepare(const FaBwdArgs a)
 // fetched by that wave alone.  A block comes in as it lies in memory except that the 64-byte groups of four keys
 // are XOR-permuted among the four 512-byte planes, so that the transposing read of a half-wave -- four keys, all
 // 32 queries, i.e. one group in each plane -- touches every LDS bank once.
-template <bool BF16, int D, bool MASKED, bool STRIDED>
+template <bool BF16, int D, bool MASKED, int LAYOUT>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaBwdArgs a)
 {
+    constexpr bool STRIDED = LAYOUT >= 1, GENERAL = LAYOUT == 2;      // (general: any length S = S_kv)
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
     typedef TileLoader<D> Loader;
@@ -816,7 +820,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     const bool active = qw < S;                    // the last block may own fewer than 256 rows
     int t0, t1, my_lo = 1, my_hi = 0;
     fa_tile_range(S, 64, a.L, a.R, q0, S - q0 < 256 ? S - q0 : 256, &t0, &t1);
-    if (active) fa_tile_range(S, 64, a.L, a.R, qw, 32, &my_lo, &my_hi);
+    if (active) fa_tile_range(S, 64, a.L, a.R, qw, GENERAL && S - qw < 32 ? S - qw : 32, &my_lo, &my_hi);
     // this head's dS blocks; this wave reads those of query block qw / 32
     const char *ds_head = reinterpret_cast<const char *>(a.ds_blocks) + (long long)(bh - head0_q) * fa_ds_blocks_per_head(S) * kDsBlockBytes;
     const int my_qb = active ? qw >> 5 : 0;
@@ -847,7 +851,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     }
     auto issue = [&](int tile, int stage) __attribute__((always_inline)) {
         const uint32_t base = lds0 + stage * STAGEB;
-        ldk.load(Kh + (size_t)tile * 64 * k_rs, base);
+        if (GENERAL && (tile + 1) * 64 > S) ldk.load_ragged(Kh + (size_t)tile * 64 * k_rs, base, S - tile * 64, k_rs * 2);
+        else ldk.load(Kh + (size_t)tile * 64 * k_rs, base);
         if (my_lo <= tile && tile <= my_hi) {
             const char *src = ds_head + fa_ds_block_index(S, my_qb, 2 * tile) * kDsBlockBytes;      // (and its neighbour 2 tile + 1)
             const uint32_t dst = base + TILEB + wave * WAVE_DS;
@@ -858,8 +863,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
     };
     // the blocks fa_bwd_dkdv wrote: its wave with the 32 keys from `key0` on visits the query tiles of this range
     auto block_written = [&](int key0) __attribute__((always_inline)) {
+        if (GENERAL && key0 >= S) return false;          // (a wave of the key-owning kernel without any key)
         int lo, hi;
-        fa_tile_range(S, 64, a.R, a.L, key0, 32, &lo, &hi);
+        fa_tile_range(S, 64, a.R, a.L, key0, GENERAL && S - key0 < 32 ? S - key0 : 32, &lo, &hi);
         return lo <= (qw >> 6) && (qw >> 6) <= hi;
     };
 
@@ -881,7 +887,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
             if (my_lo <= t && t <= my_hi) {
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
-                    if (MASKED && !block_written(64 * t + 32 * kb)) continue;       // wave-uniform
+                    if ((MASKED || GENERAL) && !block_written(64 * t + 32 * kb)) continue;       // wave-uniform
 #pragma unroll
                     for (int t2 = 0; t2 < 2; ++t2) {
                         const u32x2 lo = lds_read_tr(ds_rd[0] + (uint32_t)(kb * kDsBlockBytes + 256 * t2));
@@ -899,7 +905,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq_from_ds(const FaB
             stage = next;
         }
     }
-    if (active) {
+    if (active && (!GENERAL || qw + l32 < S)) {
         const int my_q = qw + l32;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -926,8 +932,9 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
     const int smem_dkdv_ds = smem_dkdv + (D == 128 ? (DROPOUT ? FA_PARK_DROP : ALIBI ? 2 : 1) * 32 * kBwdWaves * 64 : 0);      // + the parked fragments
     auto kq = fa_bwd_dq<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
     auto kkv = fa_bwd_dkdv<BF16, D, MASKED, LAYOUT, ALIBI, DROPOUT>;
-    // the five-product form: regular lengths (the reference's layout or a strided one)
-    constexpr bool FIVE = LAYOUT <= 1;
+    // the five-product form: regular lengths (the reference's layout or a strided one) with dropout or ALiBi, any
+    // length S = S_kv without them
+    constexpr bool FIVE = LAYOUT <= 1 || (!ALIBI && !DROPOUT);
     constexpr int FL = FIVE ? LAYOUT : 0;
     const int smem_dq_ds = kBwdStages * (TILEB + kBwdWaves * 2 * kDsBlockBytes);
     // the LDS opt-in is per (instantiation, device) and is made once, not on every launch
@@ -942,7 +949,7 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dkdv<BF16, D, MASKED, FL, ALIBI, DROPOUT, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkdv_ds);
             if (e != hipSuccess) return e;
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>),
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fa_bwd_dq_from_ds<BF16, D, MASKED, FL>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem_dq_ds);
             if (e != hipSuccess) return e;
         }
@@ -975,7 +982,7 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
             // workspace holds dS blocks for: dK, dV and the dS blocks; dQ from the blocks
             constexpr int rows_per_block = 256 / (D / 8);
             const long long n_rows = (long long)a.B * a.H * a.S;
-            hipLaunchKernelGGL((fa_bwd_prepare<BF16, D, FL == 1>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL((fa_bwd_prepare<BF16, D, FL >= 1>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0, stream, a);
             const int chunk = a.ds_heads > 0 && a.ds_heads < all_heads ? a.ds_heads : all_heads;
             for (int h0 = 0; h0 < all_heads; h0 += chunk) {
                 a.head0 = h0;
@@ -983,7 +990,7 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
                 const unsigned launch_k = grid_for((long long)a.heads * ((a.Sk + 255) / 256));
                 const unsigned launch_q = grid_for((long long)a.heads * group * ((a.S + 255) / 256));
                 hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, ALIBI, DROPOUT, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
-                hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL == 1>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
+                hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
             }
             return hipGetLastError();
         }

@@ -55,7 +55,7 @@ FA_LAYOUT_HD int fa_bwd_tr_read(int D, int lane, int db, int hi)
 // (with whole block rows the query-owning kernel's eight waves read 512 KiB apart: 0.87 ms against 0.82 on B2 H32
 // S8192 D128); inside a square the key block runs fastest, so the two blocks a query-owning wave needs per key tile
 // are neighbours.
-FA_LAYOUT_HD long long fa_ds_squares_per_side(int S) { return (S / 32 + 7) / 8; }
+FA_LAYOUT_HD long long fa_ds_squares_per_side(int S) { return ((S + 31) / 32 + 7) / 8; }
 FA_LAYOUT_HD long long fa_ds_blocks_per_head(int S) { return fa_ds_squares_per_side(S) * fa_ds_squares_per_side(S) * 64; }
 FA_LAYOUT_HD long long fa_ds_block_index(int S, int qb, int kb)
 {

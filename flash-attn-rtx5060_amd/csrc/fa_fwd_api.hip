@@ -669,12 +669,13 @@ unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p)
 }
 
 namespace {
-// what the contiguous and the strided kernels run: S a multiple of 128 and as many keys, in any storage order and
-// with any grouping of K/V heads, with dropout or with ALiBi (both at once run the general kernels)
+// as many keys as queries, in any storage order and with any grouping of K/V heads; lengths that are a multiple of
+// 128 also with dropout or with ALiBi (not both), other lengths without either
 bool five_product_shape(const fa_bwd_params *p)
 {
-    if (p->S % 128 != 0 || (p->S_kv != 0 && p->S_kv != p->S)) return false;
-    return !(p->alibi_slopes_ptr != nullptr && fa_dropout_threshold(p->dropout_prob) != 0);
+    if (p->S_kv != 0 && p->S_kv != p->S) return false;
+    const bool alibi = p->alibi_slopes_ptr != nullptr, drop = fa_dropout_threshold(p->dropout_prob) != 0;
+    return p->S % 128 == 0 ? !(alibi && drop) : !(alibi || drop);
 }
 unsigned long long ds_blocks_offset(const fa_bwd_params *p)
 {

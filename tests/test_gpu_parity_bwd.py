@@ -114,8 +114,8 @@ def test_five_product_form_against_the_fp64_oracle(fa, oracle, shape, dtype, cau
 
 
 def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
-    """Lengths a multiple of 128 with as many keys, in any storage order and with any grouping of K/V heads (the dS
-    blocks are per QUERY head), with dropout or with ALiBi; not with other lengths, nor with both options at once."""
+    """As many keys as queries, in any storage order and with any grouping of K/V heads (the dS blocks are per QUERY
+    head); lengths a multiple of 128 also with dropout or with ALiBi (not both at once), other lengths without."""
     import ctypes
     L = fa.lib()
     ok = dict(B=2, N=4, S=1024, d=128)
@@ -125,7 +125,11 @@ def test_five_product_workspace_is_offered_for_regular_lengths_only(fa):
     for same in (dict(n_kv_heads=2), dict(n_kv_heads=1), dict(strides={"q": (4 * 1024 * 128, 128, 4 * 128)}), dict(dropout_prob=0.1),
                  dict(alibi_ptr=256)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **same}))) == large, same
-    for other in (dict(S=1000), dict(S_kv=2048), dict(alibi_ptr=256, dropout_prob=0.1)):
+    ragged = dict(B=2, N=4, S=1000, d=128)
+    small_r = L.fa_bwd_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ragged)))
+    # (32 blocks of 32 queries or keys per side, in four squares of eight: as many as S = 1024 has)
+    assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**ragged))) == ((small_r + 255) // 256) * 256 + 2 * 4 * 1024 * 1024 * 2
+    for other in (dict(S=1000, dropout_prob=0.1), dict(S=1000, alibi_ptr=256), dict(S_kv=2048), dict(alibi_ptr=256, dropout_prob=0.1)):
         assert L.fa_bwd_fast_workspace_bytes(ctypes.byref(fa.make_bwd_params(**{**ok, **other}))) == 0, other
 
 
@@ -179,6 +183,27 @@ FIVE_STRIDED = [
 def test_five_product_form_in_strided_layouts_and_with_grouped_heads(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd):
     """[B,S,H,D] storage and K/V heads shared by groups of query heads: the key-owning workgroup writes the dS blocks
     of every query head of its group."""
+    five_product_case(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd, False)
+
+
+FIVE_RAGGED = [
+    # B, H, Hk, S, D, dtype, causal, wl, wr, bshd: any length with as many keys, through the general kernels
+    (1, 2, 2, 100, 64, 0, True, -1, -1, False),
+    (2, 4, 2, 333, 128, 0, True, -1, -1, False),
+    (1, 2, 1, 300, 128, 1, False, -1, -1, True),
+    (1, 2, 2, 1000, 128, 0, True, -1, -1, False),       # the last 32-key block of the last tile holds 8 keys
+    (1, 3, 3, 970, 64, 0, True, 200, -1, True),         # ... holds none: its wave of the key-owning kernel has no key
+    (1, 2, 2, 1, 128, 0, True, -1, -1, False),
+    (2, 2, 1, 33, 64, 1, False, 5, 7, False),
+    (1, 4, 2, 577, 128, 0, False, 100, 60, True),
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,D,dtype,causal,wl,wr,bshd", FIVE_RAGGED)
+def test_five_product_form_at_any_length(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd):
+    """Lengths that are not a multiple of 128 (as many keys as queries): the general kernels write and read the dS
+    blocks too.  Lanes of the key-owning kernel whose key lies past the end store zeros, 32-key blocks without any
+    key are neither written nor read, query rows past the end are masked to zero: with a NaN-filled workspace."""
     five_product_case(fa, oracle, B, H, Hk, S, D, dtype, causal, wl, wr, bshd, False)
 
 
