@@ -31,6 +31,9 @@
 #include "fa_bwd_args.h"
 #include "fa_bwd_layout.h"
 
+#ifndef FA_DS_LOOP
+#define FA_DS_LOOP 1
+#endif
 #ifndef FA_PARK_DROP
 #define FA_PARK_DROP 3
 #endif
@@ -390,7 +393,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dq(const FaBwdArgs a
 template <bool BF16, int D, bool MASKED, int LAYOUT, bool ALIBI, bool DROPOUT, bool WRITE_DS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) fa_bwd_dkdv(const FaBwdArgs a)
 {
-    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES && D == 128;
+    constexpr bool STRIDES = LAYOUT >= 1, GENERAL = LAYOUT == 2, ONE_ITEM = STRIDES && D == 128 && !(WRITE_DS && FA_DS_LOOP);
     static_assert(!WRITE_DS || LAYOUT <= 1 || (!ALIBI && !DROPOUT), "general lengths: dS blocks without ALiBi and dropout only");
     typedef Num<BF16> N;
     typedef TileReader<D> Reader;
@@ -971,11 +974,15 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
     // (The 128-wide strided and general instantiations are launched one workgroup per item only: with the item loop
     // around them they spill ten times as much, and a reload inside the tile loop waits for every tile load in
     // flight: c3's shape stored [B,S,H,D] 4.1 ms against 3.8.  The 64-wide ones have the registers for the loop.)
-    const bool uneven = (LAYOUT == 0 || D == 64) && MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
-    auto grid_for = [&](long long items) {
+    // (The kernels of the five-product form have the loop in every layout: the key-owning one keeps K^T / V^T
+    // fragments in LDS and compiles with it without spilling, or with 12 bytes outside the tile loop.)
+    const bool uneven_items = MASKED && (a.L < unbounded || a.R < unbounded) && 2LL * a.L > (long long)a.S;
+    const bool uneven = (LAYOUT == 0 || D == 64) && uneven_items;
+    auto grid_if = [&](bool snake, long long items) {
         const unsigned g = (unsigned)items;
-        return (uneven && g > resident && g < 16u * resident) ? resident : g;
+        return (snake && g > resident && g < 16u * resident) ? resident : g;
     };
+    auto grid_for = [&](long long items) { return grid_if(uneven, items); };
     if constexpr (FIVE) {
         if (a.ds_blocks != nullptr) {
             // delta and the rescaled logsumexp, for all heads at once; then, for as many heads at a time as the
@@ -987,8 +994,8 @@ hipError_t launch_bwd(const FaBwdArgs &a_in, int compute_units, hipStream_t stre
             for (int h0 = 0; h0 < all_heads; h0 += chunk) {
                 a.head0 = h0;
                 a.heads = all_heads - h0 < chunk ? all_heads - h0 : chunk;
-                const unsigned launch_k = grid_for((long long)a.heads * ((a.Sk + 255) / 256));
-                const unsigned launch_q = grid_for((long long)a.heads * group * ((a.S + 255) / 256));
+                const unsigned launch_k = grid_if(FA_DS_LOOP ? uneven_items : uneven, (long long)a.heads * ((a.Sk + 255) / 256));
+                const unsigned launch_q = grid_if(uneven_items, (long long)a.heads * group * ((a.S + 255) / 256));
                 hipLaunchKernelGGL((fa_bwd_dkdv<BF16, D, MASKED, FL, ALIBI, DROPOUT, true>), dim3(launch_k), dim3(kBwdWaves * 64), smem_dkdv_ds, stream, a);
                 hipLaunchKernelGGL((fa_bwd_dq_from_ds<BF16, D, MASKED, FL>), dim3(launch_q), dim3(kBwdWaves * 64), smem_dq_ds, stream, a);
             }

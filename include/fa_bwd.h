@@ -58,8 +58,9 @@ typedef struct fa_bwd_params {
 
 int fa_bwd_validate(const fa_bwd_params *p);
 unsigned long long fa_bwd_workspace_bytes(const fa_bwd_params *p);
-/* The workspace size that selects the five-product form, or 0 when the problem has none (it needs S a multiple
- * of 128 and as many keys; any storage order, any grouping of K/V heads, with dropout or with ALiBi, not with both): the small
+/* The workspace size that selects the five-product form, or 0 when the problem has none (it needs as many
+ * keys as queries; any storage order and grouping of K/V heads; dropout or ALiBi, not both, and only when S is a
+ * multiple of 128): the small
  * workspace plus B*N*S*S storage-type elements (B2 N32 S8192: 8.6 GB).  With it, the key-owning kernel writes every
  * dS block it forms and dQ is one product over those blocks, instead of a second recomputation of S and dP. */
 unsigned long long fa_bwd_fast_workspace_bytes(const fa_bwd_params *p);
