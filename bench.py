@@ -22,14 +22,14 @@ PEAK_TFLOPS = 2516.6   # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz: dense fp16 = bf16 
 # HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # script, each scaled by what the same counter reads for a plain 512 MiB copy kernel (FETCH_SIZE counts are
 # worth 2.000 KiB, WRITE_SIZE counts 1.000 KiB).  c3: 426.3 MB read + 136.4 MB written (runs differ by a few per
-# cent with the L2 hit rate of the K/V re-reads: 561 to 592 MB); c2 51.0 + 17.3; c4 640.9 + 136.3.
-MEASURED_HBM_BYTES = {"c3": 562.7e6, "c2": 68.3e6, "c4": 777.2e6}
+# cent with the L2 hit rate of the K/V re-reads: 561 to 592 MB); c2 51.1 + 17.3; c4 644.0 + 136.3.
+MEASURED_HBM_BYTES = {"c3": 562.7e6, "c2": 68.4e6, "c4": 780.3e6}
 TRAFFIC_SOURCE = {"c3": "profiles/fa_fwd_pipelined_c3_pmc.md", "c2": "profiles/fa_fwd_pipelined_c2_pmc.md",
                   "c4": "profiles/fa_fwd_pipelined_c4_pmc.md"}
 # the same for the backward kernels together on c3's shape (profiles/fa_bwd_c3_backward.md): the five-product form
-# 5709.2 MB read + 4747.8 MB written (8.6 GB of it the dS blocks, written once and read once), the seven-product
+# 5723.9 MB read + 4777.0 MB written (8.6 GB of it the dS blocks, written once and read once), the seven-product
 # form 1756.4 MB read + 414.9 MB written
-MEASURED_BWD_HBM_BYTES = {"c3": {"five": 10457.0e6, "seven": 2171.3e6}}
+MEASURED_BWD_HBM_BYTES = {"c3": {"five": 10500.9e6, "seven": 2171.3e6}}
 
 WORKLOADS = {
     # name: (B, H, S, D, dtype(0 fp16, 1 bf16), causal, window_left, sigma, row_fraction, row_mult, seed)
